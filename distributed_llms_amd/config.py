@@ -22,7 +22,7 @@ from typing import Any, Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2"; layer-list models: "tudilix", "gikovik"
+    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2"; layer-list models: "tudilix", "gikovik", "zebutar"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -58,7 +58,7 @@ class ModelConfig:
     @property
     def needs_state_slots(self) -> bool:
         """Sequences carry per-layer state besides paged K/V (recurrent state, convolution tails)."""
-        return self.layers is not None and self.arch == "tudilix"
+        return self.layers is not None and self.arch in ("tudilix", "zebutar")
 
     @property
     def needs_seq_index(self) -> bool:
@@ -133,6 +133,9 @@ class ModelConfig:
             if self.token_side_dim:
                 d["token_side"] = {"dim": self.token_side_dim}
             return d
+        if self.arch == "zebutar":
+            return {"architecture": "Zebutar", "layers": [dict(l) for l in self.layers], "norm": {"eps": self.norm_eps},
+                    "vocab": self.vocab_size, "width": self.hidden_size, "_dllm_name": self.name}
         if self.layers is not None:
             return {"architecture": "Tudilix", "layers": [dict(l) for l in self.layers],
                     "logit_softcap": self.logit_softcap, "norm": {"eps": self.norm_eps},
@@ -173,6 +176,8 @@ class ModelConfig:
             return ModelConfig.from_layer_list(cfg, name)
         if cfg.get("architecture") == "Gikovik":
             return _from_gikovik(cfg, name)
+        if cfg.get("architecture") == "Zebutar":
+            return _from_zebutar(cfg, name)
         mt = cfg.get("model_type", "llama")
         name = name or cfg.get("_dllm_name") or cfg.get("_name_or_path") or mt
         eos = cfg.get("eos_token_id", 2)
@@ -263,6 +268,31 @@ def _from_gikovik(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelConfi
         token_side_dim=int((cfg.get("token_side") or {}).get("dim", 0)))
 
 
+def _from_zebutar(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelConfig:
+    """A ``config.json`` with "architecture": "Zebutar": ``width``, ``vocab``, ``norm.eps``, ``layers`` (per
+    layer ``type`` "parallel", ``mixer``: ``left`` (chunked attention sizes), ``right`` (gated delta rule
+    sizes), ``left_scale``, ``right_scale``; ``mlp`` None | dense | moe)."""
+    layers = [dict(l) for l in cfg["layers"]]
+    if not layers:
+        raise ValueError("layer-list config without layers")
+    for l in layers:
+        if l["type"] != "parallel":
+            raise ValueError(f"unsupported layer type {l['type']!r} (parallel)")
+        if l.get("mlp") is not None and l["mlp"].get("kind") not in ("dense", "moe"):
+            raise ValueError(f"unsupported mlp kind {l['mlp'].get('kind')!r} (dense, moe)")
+    extra = set(cfg.get("norm", {})) - {"eps"}
+    if extra:
+        raise ValueError(f"unsupported norm options {sorted(extra)}")
+    left = [l["mixer"]["left"] for l in layers]
+    ff = [l["mlp"]["ff"] if l["mlp"]["kind"] == "dense" else l["mlp"]["expert"]["ff"] for l in layers if l.get("mlp")]
+    return ModelConfig(
+        name=name or cfg.get("_dllm_name") or "zebutar", arch="zebutar", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), intermediate_size=int(max(ff or [0])), num_layers=len(layers),
+        num_heads=max(m["heads"] for m in left), num_kv_heads=max(m["kv_heads"] for m in left),
+        head_dim=max(max(m["dim"], m["vdim"]) for m in left), max_position=1 << 30,
+        norm_eps=float(cfg["norm"]["eps"]), bos_token_id=-1, eos_token_id=-1, layers=layers)
+
+
 _LLAMA3_ROPE = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                 "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
 
@@ -336,6 +366,28 @@ PRESETS: Dict[str, ModelConfig] = {
             {"type": "latent_attention", "mixer": {"dim": 16, "heads": 4, "kv_rank": 48, "q_rank": 64, "scale": 0.25,
                                                    "vdim": 24}, "mlp": None},
         ]}, name="tiny-gikovik"),
+    "tiny-zebutar": _from_zebutar({
+        "architecture": "Zebutar", "vocab": 288, "width": 96, "norm": {"eps": 1e-6},
+        "layers": [
+            {"type": "parallel", "mixer": {
+                "left": {"dim": 24, "vdim": 40, "heads": 4, "kv_heads": 2, "mask": {"size": 24}, "scale": 0.2,
+                         "rot": {"base": 10000.0, "dims": 16}},
+                "right": {"conv": 4, "dim": 16, "vdim": 24, "heads": 4, "kv_heads": 2},
+                "left_scale": 0.9, "right_scale": 0.7},
+             "mlp": {"kind": "dense", "ff": 160}},
+            {"type": "parallel", "mixer": {
+                "left": {"dim": 16, "vdim": 16, "heads": 3, "kv_heads": 1, "mask": {"size": 10}, "scale": 0.3,
+                         "rot": {"base": 500.0, "dims": 16}},
+                "right": {"conv": 2, "dim": 40, "vdim": 72, "heads": 2, "kv_heads": 2},
+                "left_scale": 1.1, "right_scale": 0.6},
+             "mlp": {"kind": "moe", "expert": {"ff": 48}, "shared": {"ff": 64}, "router": {"experts": 6, "top": 2}}},
+            {"type": "parallel", "mixer": {
+                "left": {"dim": 24, "vdim": 40, "heads": 4, "kv_heads": 4, "mask": {"size": 33}, "scale": 0.2,
+                         "rot": {"base": 10000.0, "dims": 8}},
+                "right": {"conv": 3, "dim": 16, "vdim": 24, "heads": 4, "kv_heads": 1},
+                "left_scale": 1.0, "right_scale": 1.0},
+             "mlp": None},
+        ]}, name="tiny-zebutar"),
     "tiny-gpt2": ModelConfig(
         name="tiny-gpt2", arch="gpt2", vocab_size=512, hidden_size=128,
         intermediate_size=512, num_layers=4, num_heads=2, num_kv_heads=2, head_dim=64,

@@ -2,7 +2,8 @@
 // (ops/seqmix.py window_attention): caches k [NB, G, BS, D] (one row per key), v [NB, G, Dv, BS]
 // (transposed inside a block: 8 keys of one value channel are one 16-byte load),
 // query head h reads K/V head h / (H / G), a query at position p sees the keys j of its sequence with
-// 0 <= p - j < window; `sinks` (float32 [H], or null) adds exp(sink_h) to head h's softmax denominator
+// 0 <= p - j < window and, with `chunk` > 0, floor(j / chunk) = floor(p / chunk) (attention inside fixed
+// chunks of positions); `sinks` (float32 [H], or null) adds exp(sink_h) to head h's softmax denominator
 // (a learned per-head logit that takes part in the normalisation only).  Scores, softmax weights and the weighted sum are float32; T is the storage
 // type (bf16 or float).  Head sizes, window and block size are runtime values.
 //
@@ -26,6 +27,15 @@
 namespace dllm {
 
 template <typename T> __device__ __forceinline__ float wld(const T* p) { return (float)*p; }
+
+// Oldest key position a query at `pos` sees: inside its window and -- with chunk > 0 -- inside its own
+// chunk of `chunk` positions, chunks counted from position 0 of the sequence (a query never looks across
+// a chunk border, wherever the prompt was cut for processing).  Not decreasing in pos.
+__device__ __forceinline__ int win_lo(int pos, int window, int chunk) {
+  int lo = max(0, pos - window + 1);
+  if (chunk > 0) lo = max(lo, pos - pos % chunk);
+  return lo;
+}
 
 constexpr int kWinTile = 256;     // keys per tile = threads per workgroup
 constexpr int kWinMaxAcc = 2;     // value channels per thread: Dv <= 256 * kWinMaxAcc
@@ -77,7 +87,7 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
     void* __restrict__ out_, const void* __restrict__ q_, const void* __restrict__ k_cache_,
     const void* __restrict__ v_cache_, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int t0, int H, int G, int D, int Dv,
-    int bs, int window, float scale, const float* __restrict__ sinks) {
+    int bs, int window, int chunk, float scale, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   float* qs = lds;                       // [D]
   float* p = qs + D;                     // [kWinTile]
@@ -87,7 +97,7 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
   const int t = t0 + blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int g = h / (H / G);
   const int pos = positions[t], b = tok_seq[t];
-  const int lo = max(0, pos - window + 1);
+  const int lo = win_lo(pos, window, chunk);
   const T* q = (const T*)q_ + ((size_t)t * H + h) * D;
   const T* kc = (const T*)k_cache_;
   const T* vc = (const T*)v_cache_;
@@ -162,21 +172,21 @@ static size_t win_row_lds(int D, int Dv) {
 
 static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t positions, uintptr_t tok_seq, int t0, int rows, int H, int G, int D,
-                        int Dv, int bs, int window, float scale, uintptr_t sinks, int f32, uintptr_t stream) {
+                        int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int f32, uintptr_t stream) {
   DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0 && Dv <= kWinTile * kWinMaxAcc, "window attention heads");
-  DLLM_HOST_CHECK(bs > 0 && window >= 1 && max_blocks > 0 && H <= 65535, "window attention sizes");
+  DLLM_HOST_CHECK(bs > 0 && window >= 1 && chunk >= 0 && max_blocks > 0 && H <= 65535, "window attention sizes");
   const size_t lds = win_row_lds(D, Dv);
   DLLM_HOST_CHECK(lds <= 64 * 1024, "window attention head size");
   if (f32)
     hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_row_kernel<float>), dim3(rows, H), dim3(kWinTile), lds,
                        (hipStream_t)stream, (void*)out, (const void*)q, (const void*)k_cache, (const void*)v_cache,
                        (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, t0,
-                       H, G, D, Dv, bs, window, scale, (const float*)sinks);
+                       H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks);
   else
     hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_row_kernel<bf16>), dim3(rows, H), dim3(kWinTile), lds,
                        (hipStream_t)stream, (void*)out, (const void*)q, (const void*)k_cache, (const void*)v_cache,
                        (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, t0,
-                       H, G, D, Dv, bs, window, scale, (const float*)sinks);
+                       H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks);
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
@@ -216,7 +226,7 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int nseq, int nqt, int H, int G,
-    int D, int Dv, int bs, int window, float scale, const float* __restrict__ sinks, int sub) {
+    int D, int Dv, int bs, int window, int chunk, float scale, const float* __restrict__ sinks, int sub) {
   constexpr int kQT = QT, kTQ = 64 * QT;
   constexpr int DP = 32 * NQK, KROW = DP + kPad, VROW = kTK + kPad;
   constexpr int KPT = (kTK * (DP / 8) + 255) / 256, VPT = (16 * NDV * (kTK / 8) + 255) / 256;   // 16-byte pieces per thread
@@ -244,7 +254,7 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   const int bsh = __ffs(bs) - 1;                                       // bs is a power of two here
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   // this lane's two queries (MFMA columns of the wave's two column tiles)
-  int ql[kQT], qpos[kQT];
+  int ql[kQT], qpos[kQT], qlo[kQT];
   bool qok[kQT];
   bf16x8 qf[kQT][NQK];
 #pragma unroll
@@ -252,6 +262,7 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     ql[c2] = q0 + wave * 16 * kQT + c2 * 16 + col;
     qok[c2] = ql[c2] < n;
     qpos[c2] = start + min(ql[c2], n - 1);
+    qlo[c2] = win_lo(qpos[c2], window, chunk);
     const bf16* qrow = q + ((size_t)(lo_t + min(ql[c2], n - 1)) * H + h) * D;
 #pragma unroll
     for (int s2 = 0; s2 < NQK; ++s2) {
@@ -276,7 +287,7 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
 #pragma unroll
   for (int c2 = 0; c2 < kQT; ++c2) m[c2] = -INFINITY, l[c2] = 0.f;
   const int last_pos = start + min(q0 + kTQ, n) - 1;                   // newest key any query of the tile sees
-  const int first_pos = max(0, start + q0 - window + 1);               // oldest
+  const int first_pos = win_lo(start + q0, window, chunk);             // oldest
   const int d8 = D >> 3;
   const float sc2 = scale * kLog2e;
   bf16x8 kreg[KPT], vreg[VPT];
@@ -325,10 +336,10 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   };
   // keys the wave's queries see: [wlo, whi]
   const int wq0 = q0 + wave * 16 * kQT;
-  const int whi = start + min(wq0 + 16 * kQT - 1, n - 1), wlo = max(0, start + wq0 - window + 1);
+  const int whi = start + min(wq0 + 16 * kQT - 1, n - 1), wlo = win_lo(start + wq0, window, chunk);
   // a tile whose keys every query of the wave sees needs no mask: all keys <= the wave's first query's
   // position and inside the window of its last one
-  const int full_hi = start + wq0, full_lo = whi - window + 1;
+  const int full_hi = start + wq0, full_lo = win_lo(whi, window, chunk);
   const bool wave_full = wq0 + 16 * kQT <= n;
   const int kfirst = first_pos & ~(kTK - 1);
   fetch(kfirst);
@@ -370,7 +381,7 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
           for (int i = 0; i < 8; ++i) {
             const int kp = k0 + 8 * grp + i;
             const float sv = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
-            const bool ok = qok[c2] && kp <= qpos[c2] && qpos[c2] - kp < window;
+            const bool ok = qok[c2] && kp <= qpos[c2] && kp >= qlo[c2];
             p[i] = ok ? sv : -INFINITY;
             cm = fmaxf(cm, p[i]);
           }
@@ -435,7 +446,8 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
 template <int NQK, int NDV, int QT>
 static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t cu, uintptr_t positions, int seq0, int nseq, int max_q_len, int H,
-                        int G, int D, int Dv, int bs, int window, float scale, uintptr_t sinks, uintptr_t stream) {
+                        int G, int D, int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks,
+                        uintptr_t stream) {
   constexpr int kTQ = 64 * QT;
   const int nqt = (max_q_len + kTQ - 1) / kTQ;
   const int pairs = nseq * G, per_pair = nqt * (H / G);
@@ -445,7 +457,7 @@ static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
   hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV, QT>), dim3((unsigned)(per_xcd * 8)),
                      dim3(256), 0, (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
                      (const bf16*)v_cache, (const int32_t*)block_tables, max_blocks, (const int32_t*)cu,
-                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, scale, (const float*)sinks, sub);
+                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks, sub);
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
@@ -463,7 +475,7 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int H, int G, int D, int Dv, int bs,
-    int window, float scale, const float* __restrict__ sinks, int hpw, int splits, float* __restrict__ ws) {
+    int window, int chunk, float scale, const float* __restrict__ sinks, int hpw, int splits, float* __restrict__ ws) {
   constexpr int DVP = 16 * NDV;
   __shared__ float so[kDW][16][DVP + 1];
   __shared__ float sml[kDW][2][16];
@@ -475,7 +487,7 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   const int hb = g * R + hpw * part, nh = min(hpw, R - hpw * part);    // first head and heads of this workgroup
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, grp = lane >> 4;
   const int pos = positions[t], b = tok_seq[t];
-  const int lo = max(0, pos - window + 1);
+  const int lo = win_lo(pos, window, chunk);
   const int bsh = __ffs(bs) - 1;                     // bs is a power of two here
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   bf16x8 qf[NQK];
@@ -640,7 +652,7 @@ __global__ void __launch_bounds__(64) window_attn_merge_kernel(bf16* __restrict_
 template <int NQK, int NDV>
 static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                           int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
-                          int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
+                          int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int splits, uintptr_t ws,
                           uintptr_t stream) {
   // heads per workgroup: 16 (all MFMA columns) when rows x K/V heads x key runs fill the chip, else halved
   // until about half the CUs have a workgroup -- the keys are re-read from L2, the columns left idle cost
@@ -654,7 +666,7 @@ static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr
                      dim3(rows, G * ((R + hpw - 1) / hpw), splits), dim3(64 * kDW), 0,
                      (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
                      (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, H, G,
-                     D, Dv, bs, window, scale, (const float*)sinks, hpw, splits, (float*)ws);
+                     D, Dv, bs, window, chunk, scale, (const float*)sinks, hpw, splits, (float*)ws);
   DLLM_HIP_CHECK(hipGetLastError());
   if (splits > 1) {
     hipLaunchKernelGGL(window_attn_merge_kernel, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, (bf16*)out,
@@ -675,14 +687,14 @@ static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs) {
 // kernel only; the row kernel ignores it).
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
-                           int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
+                           int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int splits, uintptr_t ws,
                            int f32, uintptr_t stream) {
   if (rows <= 0) return;
   if (win_mfma_ok(f32, H, G, D, Dv, bs) && (long)G * ((H / G + 1) / 2) <= 65535) {
-    DLLM_HOST_CHECK(window >= 1 && max_blocks > 0, "window attention sizes");
+    DLLM_HOST_CHECK(window >= 1 && chunk >= 0 && max_blocks > 0, "window attention sizes");
 #define WIN_DEC(NQK, NDV)                                                                                       \
   launch_decode<NQK, NDV>(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, rows, H, G, D, Dv, \
-                          bs, window, scale, sinks, splits, ws, stream)
+                          bs, window, chunk, scale, sinks, splits, ws, stream)
     if (D <= 64 && Dv <= 64) WIN_DEC(2, 4);
     else if (D <= 128 && Dv <= 128) WIN_DEC(4, 8);
     else WIN_DEC(8, 16);
@@ -690,23 +702,23 @@ void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintpt
     return;
   }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, 0, rows, H, G, D, Dv, bs, window,
-              scale, sinks, f32, stream);
+              chunk, scale, sinks, f32, stream);
 }
 
 // Prompt chunks: tokens [t0 .. tokens) of sequences [seq0, seqs).
 void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                             int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
-                            int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, float scale,
-                            uintptr_t sinks, int f32, uintptr_t stream) {
+                            int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, int chunk,
+                            float scale, uintptr_t sinks, int f32, uintptr_t stream) {
   // tokens of the decode rows come first: one per sequence before seq0
   const int t0 = seq0;
   if (tokens <= t0) return;
   if (win_mfma_ok(f32, H, G, D, Dv, bs) && seqs > seq0 && max_q_len > 1) {
     DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && H <= 65535 && seqs - seq0 <= 65535, "window attention heads");
-    DLLM_HOST_CHECK(bs > 0 && window >= 1 && max_blocks > 0, "window attention sizes");
+    DLLM_HOST_CHECK(bs > 0 && window >= 1 && chunk >= 0 && max_blocks > 0, "window attention sizes");
 #define WIN_TILE(NQK, NDV, QT)                                                                                  \
   launch_tile<NQK, NDV, QT>(out, q, k_cache, v_cache, block_tables, max_blocks, cu, positions, seq0, seqs - seq0, \
-                            max_q_len, H, G, D, Dv, bs, window, scale, sinks, stream)
+                            max_q_len, H, G, D, Dv, bs, window, chunk, scale, sinks, stream)
     if (D <= 64 && Dv <= 64) WIN_TILE(2, 4, 1);
     else if (D <= 128 && Dv <= 128) WIN_TILE(4, 8, 1);
     else WIN_TILE(8, 16, 2);     // wide heads: 2b-size latent attention prompts 32 x 1024 +7 %, 4 x 4096 +29 % over QT = 1
@@ -714,7 +726,7 @@ void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintp
     return;
   }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, t0, tokens - t0, H, G, D, Dv, bs,
-              window, scale, sinks, f32, stream);
+              window, chunk, scale, sinks, f32, stream);
 }
 
 }  // namespace dllm

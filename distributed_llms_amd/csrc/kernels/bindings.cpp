@@ -62,6 +62,11 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("moe_route_groups", &dllm::moe_route_groups);
   m.def("moe_router_groups", &dllm::moe_router_groups);
   m.def("relu_sq", &dllm::relu_sq);
+  m.def("sm_embed_norm", &dllm::sm_embed_norm);
+  m.def("sm_rownorm_rope", &dllm::sm_rownorm_rope);
+  m.def("dr_prep", &dllm::dr_prep);
+  m.def("dr_scan", &dllm::dr_scan);
+  m.def("dr_out_norm", &dllm::dr_out_norm);
   m.def("moe_combine_gated", &dllm::moe_combine_gated);
   m.def("p2p_inbox_bytes", &dllm::p2p_inbox_bytes);
   m.def("p2p_standin", &dllm::p2p_standin);

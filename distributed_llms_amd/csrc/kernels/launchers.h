@@ -71,13 +71,16 @@ void paged_attention_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uint
 // are float (else bf16)
 void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int width, int vocab, int f32,
                   uintptr_t stream);
+void sm_embed_norm(uintptr_t x, uintptr_t h, uintptr_t ids, uintptr_t table, uintptr_t w, int tokens, int width,
+                   int vocab, float eps, float offset, int f32, uintptr_t stream);
 void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, float eps, float offset, int f32,
                  uintptr_t stream);
 void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
-                      int rows, int width, float eps, float mult, float offset, int f32, uintptr_t stream);
+                      int rows, int width, float eps, float mult, float offset, uintptr_t o2, float s1, float s2,
+                      int f32, uintptr_t stream);
 void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,
                     uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
-                    int tokens, int seqs, int C, int taps, int f32, int out_f32, uintptr_t stream);
+                    int tokens, int seqs, int C, int taps, int f32, int out_f32, int act, uintptr_t stream);
 void sm_rglru_gates(uintptr_t a, uintptr_t g, uintptr_t u, uintptr_t ra_t, uintptr_t ra_b, uintptr_t ri_t,
                     uintptr_t ri_b, uintptr_t lam, int tokens, int nb, int bw, float scale, int f32,
                     uintptr_t stream);
@@ -92,14 +95,17 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
                   uintptr_t v_cache, uintptr_t slot_mapping, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq,
                   uintptr_t slots, int tokens, int seqs, int H, int G, int D, int Dv, int taps, int bs, int f32,
                   uintptr_t stream);
+void sm_rownorm_rope(uintptr_t q_out, uintptr_t qkv, long ld, int col0, uintptr_t q_norm, uintptr_t k_norm,
+                     uintptr_t freqs, int nrot, float eps, uintptr_t k_cache, uintptr_t v_cache, uintptr_t slot_mapping,
+                     uintptr_t positions, int tokens, int H, int G, int D, int Dv, int bs, int f32, uintptr_t stream);
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
-                           int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
+                           int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int splits, uintptr_t ws,
                            int f32, uintptr_t stream);
 void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                             int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
-                            int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, float scale,
-                            uintptr_t sinks, int f32, uintptr_t stream);
+                            int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, int chunk,
+                            float scale, uintptr_t sinks, int f32, uintptr_t stream);
 // latent attention input stage and parallel layers on a float32 stream (latent.hip)
 void lat_prep(uintptr_t cq, uintptr_t down, long ld, int q_off, int q_rank, uintptr_t qn_w, int c_off, int rank,
               uintptr_t cn_w, int r_off, int rot_dim, uintptr_t freqs, int nfreq, uintptr_t positions,
@@ -121,12 +127,20 @@ void side_gate(uintptr_t g, uintptr_t z, uintptr_t table, uintptr_t ids, int tok
                int dim, int f32, uintptr_t stream);
 // grouped-choice router, squared ReLU and the weighted sum with a gated shared expert (moe.hip)
 void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, int E, int k, int groups, int keep,
-                      float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts, uintptr_t offsets,
-                      uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream);
+                      float scale, int softmax_top, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts,
+                      uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream);
 void moe_router_groups(uintptr_t x, uintptr_t w, int K, int rows, uintptr_t logits, uintptr_t correction, int T, int E,
-                       int k, int groups, int keep, float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts,
-                       uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, int f32, uintptr_t stream);
+                       int k, int groups, int keep, float scale, int softmax_top, uintptr_t topk_w, uintptr_t topk_ids,
+                       uintptr_t counts, uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, int f32,
+                       uintptr_t stream);
 void relu_sq(uintptr_t y, long n, int f32, uintptr_t stream);
+// gated delta rule (delta.hip): everything float32 but the gate, the norm weight and the normed output
+void dr_prep(uintptr_t u, long ld, uintptr_t ab, long ldab, int bcol, uintptr_t a_log, uintptr_t dt_bias, uintptr_t bd,
+             int tokens, int H, int G, int dim, float qscale, float unit_eps, int f32, uintptr_t stream);
+void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t state, uintptr_t cu, uintptr_t positions,
+             uintptr_t slots, int seqs, int H, int G, int dim, int vdim, uintptr_t stream);
+void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
+                 int vdim, float eps, float out_scale, int f32, uintptr_t stream);
 void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,
                        uintptr_t gate_logits, long gate_ld, int T, int H, int k, int f32, uintptr_t stream);
 

@@ -374,21 +374,28 @@ void moe_combine(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t i
 // s, normalised to sum one (+ 1e-20 in the divisor) and multiplied by `scale`.  One thread per token, 128 tokens per
 // workgroup; moe_scatter_wide_kernel (one workgroup, LDS counters) then makes the counts / offsets /
 // expert-sorted slot lists that the grouped GEMMs and the combine read.
+// `softmax_top` != 0 is the other router form: selection ranks the logits plus `correction` (here a bias
+// that is part of the logit), and the mixing weights are the softmax over the selected logits only,
+// times `scale`; groups do not apply.
 constexpr int kMaxGroups = 64;
 constexpr int kMaxChoiceExperts = 256;
 
 // one token's selection from its E logits `lg`
 template <int EMAX>
 __device__ __forceinline__ void choose_groups(const float* __restrict__ lg, const float* __restrict__ correction, int E,
-                                              int k, int groups, int keep, float scale, float* __restrict__ tw,
-                                              int* __restrict__ ti) {
+                                              int k, int groups, int keep, float scale, int softmax_top,
+                                              float* __restrict__ tw, int* __restrict__ ti) {
   const int gsz = E / groups;
   float sc[EMAX], ch[EMAX];
   for (int e = 0; e < E; ++e) {
-    sc[e] = 1.0f / (1.0f + expf(-lg[e]));
-    ch[e] = sc[e] + (correction ? correction[e] : 0.f);
+    if (softmax_top) {
+      sc[e] = ch[e] = lg[e] + (correction ? correction[e] : 0.f);
+    } else {
+      sc[e] = 1.0f / (1.0f + expf(-lg[e]));
+      ch[e] = sc[e] + (correction ? correction[e] : 0.f);
+    }
   }
-  if (keep < groups) {
+  if (keep < groups && !softmax_top) {
     float gs[kMaxGroups];
     for (int g = 0; g < groups; ++g) {
       float a = -INFINITY, b = -INFINITY;          // top two of the block
@@ -421,22 +428,22 @@ __device__ __forceinline__ void choose_groups(const float* __restrict__ lg, cons
       if (!taken && (best < 0 || ch[e] > bv)) { bv = ch[e]; best = e; }
     }
     ids[j] = best;
-    tot += sc[best];
+    tot += softmax_top ? expf(sc[best] - sc[ids[0]]) : sc[best];      // ids[0] holds the largest logit
   }
   for (int j = 0; j < k; ++j) {
     ti[j] = ids[j];
-    tw[j] = sc[ids[j]] / (tot + 1e-20f) * scale;
+    tw[j] = softmax_top ? expf(sc[ids[j]] - sc[ids[0]]) / tot * scale : sc[ids[j]] / (tot + 1e-20f) * scale;
   }
 }
 
 template <int EMAX>
 __global__ void __launch_bounds__(128) moe_choice_groups_kernel(
     const float* __restrict__ logits, long ld, const float* __restrict__ correction, int T, int E, int k, int groups,
-    int keep, float scale, float* __restrict__ topk_w, int* __restrict__ topk_ids) {
+    int keep, float scale, int softmax_top, float* __restrict__ topk_w, int* __restrict__ topk_ids) {
   const int t = blockIdx.x * 128 + threadIdx.x;
   if (t >= T) return;
-  choose_groups<EMAX>(logits + (size_t)t * ld, correction, E, k, groups, keep, scale, topk_w + (size_t)t * k,
-                      topk_ids + (size_t)t * k);
+  choose_groups<EMAX>(logits + (size_t)t * ld, correction, E, k, groups, keep, scale, softmax_top,
+                      topk_w + (size_t)t * k, topk_ids + (size_t)t * k);
 }
 
 // Few tokens (decode steps): the router product and the selection in one launch, a workgroup per token.
@@ -445,8 +452,8 @@ __global__ void __launch_bounds__(128) moe_choice_groups_kernel(
 template <typename TX, int EMAX>
 __global__ void __launch_bounds__(256) moe_router_groups_kernel(
     const TX* __restrict__ x, const float* __restrict__ w, int K, int rows, float* __restrict__ logits,
-    const float* __restrict__ correction, int E, int k, int groups, int keep, float scale, float* __restrict__ topk_w,
-    int* __restrict__ topk_ids) {
+    const float* __restrict__ correction, int E, int k, int groups, int keep, float scale, int softmax_top,
+    float* __restrict__ topk_w, int* __restrict__ topk_ids) {
   __shared__ float lg[kMaxChoiceExperts + 8];
   const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const TX* xr = x + (size_t)t * K;
@@ -472,7 +479,8 @@ __global__ void __launch_bounds__(256) moe_router_groups_kernel(
   }
   __syncthreads();
   if (threadIdx.x == 0)
-    choose_groups<EMAX>(lg, correction, E, k, groups, keep, scale, topk_w + (size_t)t * k, topk_ids + (size_t)t * k);
+    choose_groups<EMAX>(lg, correction, E, k, groups, keep, scale, softmax_top, topk_w + (size_t)t * k,
+                        topk_ids + (size_t)t * k);
 }
 
 __global__ void __launch_bounds__(1024) moe_scatter_wide_kernel(const int* __restrict__ topk_ids, int T, int E, int k,
@@ -502,8 +510,8 @@ __global__ void __launch_bounds__(1024) moe_scatter_wide_kernel(const int* __res
 }
 
 void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, int E, int k, int groups, int keep,
-                      float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts, uintptr_t offsets,
-                      uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream) {
+                      float scale, int softmax_top, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts,
+                      uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream) {
   DLLM_HOST_CHECK(E >= 1 && E <= kMaxChoiceExperts && ld >= E, "1 <= experts <= 256");
   DLLM_HOST_CHECK(k >= 1 && k <= 16 && k <= E, "1 <= top <= min(16, experts)");
   DLLM_HOST_CHECK(groups >= 1 && groups <= kMaxGroups && E % groups == 0 && keep >= 1 && keep <= groups &&
@@ -513,7 +521,8 @@ void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, in
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define ROUTE_G(EMAX)                                                                                              \
   hipLaunchKernelGGL(moe_choice_groups_kernel<EMAX>, dim3((T + 127) / 128), dim3(128), 0, s, (const float*)logits, \
-                     ld, (const float*)correction, T, E, k, groups, keep, scale, (float*)topk_w, (int*)topk_ids)
+                     ld, (const float*)correction, T, E, k, groups, keep, scale, softmax_top, (float*)topk_w,    \
+                     (int*)topk_ids)
   if (E <= 16) ROUTE_G(16);
   else if (E <= 64) ROUTE_G(64);
   else ROUTE_G(256);
@@ -525,8 +534,9 @@ void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, in
 }
 
 void moe_router_groups(uintptr_t x, uintptr_t w, int K, int rows, uintptr_t logits, uintptr_t correction, int T, int E,
-                       int k, int groups, int keep, float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts,
-                       uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, int f32, uintptr_t stream) {
+                       int k, int groups, int keep, float scale, int softmax_top, uintptr_t topk_w, uintptr_t topk_ids,
+                       uintptr_t counts, uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, int f32,
+                       uintptr_t stream) {
   DLLM_HOST_CHECK(E >= 1 && E <= kMaxChoiceExperts && rows >= E && rows <= kMaxChoiceExperts + 8 && K > 0,
                   "1 <= experts <= 256, up to 8 further rows");
   DLLM_HOST_CHECK(k >= 1 && k <= 16 && k <= E, "1 <= top <= min(16, experts)");
@@ -537,8 +547,8 @@ void moe_router_groups(uintptr_t x, uintptr_t w, int K, int rows, uintptr_t logi
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 #define ROUTER_G(TX, EMAX)                                                                                       \
   hipLaunchKernelGGL((moe_router_groups_kernel<TX, EMAX>), dim3(T), dim3(256), 0, s, (const TX*)x, (const float*)w, \
-                     K, rows, (float*)logits, (const float*)correction, E, k, groups, keep, scale, (float*)topk_w,  \
-                     (int*)topk_ids)
+                     K, rows, (float*)logits, (const float*)correction, E, k, groups, keep, scale, softmax_top,     \
+                     (float*)topk_w, (int*)topk_ids)
   if (f32) { if (E <= 16) ROUTER_G(float, 16); else if (E <= 64) ROUTER_G(float, 64); else ROUTER_G(float, 256); }
   else { if (E <= 16) ROUTER_G(bf16, 16); else if (E <= 64) ROUTER_G(bf16, 64); else ROUTER_G(bf16, 256); }
 #undef ROUTER_G

@@ -36,6 +36,41 @@ void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int
               (const void*)table, width, vocab);
 }
 
+// --------------------------------------------------------------------------- embedding + RMS norm -> f32 stream
+// x = e / sqrt(mean(e^2) + eps) * (offset + w) for e = table[id], as the float32 stream and -- when h is
+// given -- also in the activation type (the input of a first sublayer that reads the stream unnormed).
+template <typename T>
+__global__ void __launch_bounds__(256) sm_embed_norm_kernel(float* __restrict__ x, void* __restrict__ h_,
+                                                            const int32_t* __restrict__ ids,
+                                                            const void* __restrict__ table_, const void* __restrict__ w_,
+                                                            int width, int vocab, float eps, float offset) {
+  __shared__ float red[16];
+  const T* table = (const T*)table_;
+  const T* w = (const T*)w_;
+  int id = ids[blockIdx.x];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* src = table + (size_t)id * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) { const float v = ldf(src + i); ss += v * v; }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  float* dst = x + (size_t)blockIdx.x * width;
+  T* h = h_ ? (T*)h_ + (size_t)blockIdx.x * width : nullptr;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = ldf(src + i) * inv * (offset + ldf(w + i));
+    dst[i] = v;
+    if (h) stf(h + i, v);
+  }
+}
+
+void sm_embed_norm(uintptr_t x, uintptr_t h, uintptr_t ids, uintptr_t table, uintptr_t w, int tokens, int width,
+                   int vocab, float eps, float offset, int f32, uintptr_t stream) {
+  if (tokens <= 0) return;
+  DLLM_HOST_CHECK(width > 0 && vocab > 0 && x && w, "embed_norm arguments");
+  SM_DISPATCH(f32, sm_embed_norm_kernel, dim3(tokens), dim3(256), 0, stream, (float*)x, (void*)h, (const int32_t*)ids,
+              (const void*)table, (const void*)w, width, vocab, eps, offset);
+}
+
 // --------------------------------------------------------------------------- RMS norm of an f32 row
 // y = x * rsqrt(mean(x^2) + eps) * (offset + w); one workgroup per row, V elements per lane and step.
 template <typename T, int V>
@@ -74,16 +109,20 @@ void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, flo
 }
 
 // --------------------------------------------------------------------------- close of a sublayer
-// x += mult * rms_norm(o + bias) * (offset + w_post);  h = rms_norm(x) * (offset + w_next) when w_next
+// x += mult * rms_norm(v) * (offset + w_post) with v = o + bias, or v = s1 o + s2 o2 when a second input is
+// given (two mixers side by side);  h = rms_norm(x) * (offset + w_next) when w_next, else, when h is
+// given, the new stream itself in the activation type (a following sublayer that reads x unnormed)
 // (offset 1: weights stored around zero; 0: plain weights).
 template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict__ x, const void* __restrict__ o_,
                                                                const void* __restrict__ bias_,
                                                                const void* __restrict__ wp_,
                                                                const void* __restrict__ wn_, void* __restrict__ h_,
-                                                               int width, float eps, float mult, float offset) {
+                                                               int width, float eps, float mult, float offset,
+                                                               const void* __restrict__ o2_, float s1, float s2) {
   __shared__ float red[16];
   const T* o = (const T*)o_ + (size_t)blockIdx.x * width;
+  const T* o2 = o2_ ? (const T*)o2_ + (size_t)blockIdx.x * width : nullptr;
   const T* bias = (const T*)bias_;
   const T* wp = (const T*)wp_;
   const T* wn = (const T*)wn_;
@@ -92,6 +131,11 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
   for (int i = threadIdx.x * V; i < width; i += 256 * V) {
     float v[V], bb[V];
     ldv<V>(o + i, v);
+    if (o2) {
+      ldv<V>(o2 + i, bb);
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = s1 * v[j] + s2 * bb[j];
+    }
     if (bias) {
       ldv<V>(bias + i, bb);
 #pragma unroll
@@ -102,10 +146,15 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  float s2 = 0.f;
+  float sq = 0.f;
   for (int i = threadIdx.x * V; i < width; i += 256 * V) {
     float v[V], bb[V], g[V], xv[V];
     ldv<V>(o + i, v);
+    if (o2) {
+      ldv<V>(o2 + i, bb);
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = s1 * v[j] + s2 * bb[j];
+    }
     if (bias) {
       ldv<V>(bias + i, bb);
 #pragma unroll
@@ -116,13 +165,14 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
 #pragma unroll
     for (int j = 0; j < V; ++j) {
       xv[j] = xv[j] + mult * (v[j] * inv * (offset + g[j]));
-      s2 += xv[j] * xv[j];
+      sq += xv[j] * xv[j];
     }
     stv<V>(xr + i, xv);
+    if (!wn && h_) stv<V>((T*)h_ + (size_t)blockIdx.x * width + i, xv);
   }
   if (!wn) return;
-  s2 = block_sum(s2, red);
-  const float inv2 = 1.0f / sqrtf(s2 / (float)width + eps);
+  sq = block_sum(sq, red);
+  const float inv2 = 1.0f / sqrtf(sq / (float)width + eps);
   T* h = (T*)h_ + (size_t)blockIdx.x * width;
   for (int i = threadIdx.x * V; i < width; i += 256 * V) {      // each lane re-reads what it wrote itself
     float xv[V], g[V];
@@ -135,11 +185,13 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
 }
 
 void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
-                      int rows, int width, float eps, float mult, float offset, int f32, uintptr_t stream) {
+                      int rows, int width, float eps, float mult, float offset, uintptr_t o2, float s1, float s2,
+                      int f32, uintptr_t stream) {
   if (rows <= 0) return;
   DLLM_HOST_CHECK(width > 0 && (!w_next || h), "post_norm_add arguments");
   SM_DISPATCH_V(f32, width % 8 == 0, sm_post_norm_add_kernel, dim3(rows), dim3(256), 0, stream, (float*)x,
-                (const void*)o, (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult, offset);
+                (const void*)o, (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult,
+                offset, (const void*)o2, s1, s2);
 }
 
 // --------------------------------------------------------------------------- causal convolution with state
@@ -173,7 +225,8 @@ __global__ void __launch_bounds__(256) sm_causal_conv_kernel(void* __restrict__ 
                                                              const int32_t* __restrict__ cu,
                                                              const int32_t* __restrict__ positions,
                                                              const int32_t* __restrict__ tok_seq,
-                                                             const int32_t* __restrict__ slots, int C, int taps) {
+                                                             const int32_t* __restrict__ slots, int C, int taps,
+                                                             int act) {
   const int t = blockIdx.x;
   const int b = tok_seq[t];
   const int tl = t - cu[b], pos = positions[t];
@@ -194,6 +247,10 @@ __global__ void __launch_bounds__(256) sm_causal_conv_kernel(void* __restrict__ 
       ldv<V>(w + (size_t)j * C + c, wv);
 #pragma unroll
       for (int e = 0; e < V; ++e) acc[e] += wv[e] * (xv[e] + ib[e]);
+    }
+    if (act == 1) {                                  // silu, in float32 with the exact exponential
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
     }
     stv<V>(y + c, acc);
   }
@@ -236,9 +293,9 @@ static void launch_conv_state(uintptr_t state, uintptr_t u, long stride, uintptr
 
 void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,
                     uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
-                    int tokens, int seqs, int C, int taps, int f32, int out_f32, uintptr_t stream) {
+                    int tokens, int seqs, int C, int taps, int f32, int out_f32, int act, uintptr_t stream) {
   if (tokens <= 0 || seqs <= 0) return;
-  DLLM_HOST_CHECK(C > 0 && taps >= 1 && stride >= C, "conv sizes");
+  DLLM_HOST_CHECK(C > 0 && taps >= 1 && stride >= C && (act == 0 || act == 1), "conv sizes");
   const int esz = f32 ? 4 : 2;
   const int vec = C % 8 == 0 && stride % 8 == 0 && (u % (8 * esz)) == 0;
   const int per = 256 * (vec ? 8 : 1);
@@ -247,7 +304,7 @@ void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_
 #define SM_CONV(T, OT, V)                                                                                    \
   hipLaunchKernelGGL(HIP_KERNEL_NAME(sm_causal_conv_kernel<T, OT, V>), grid, dim3(256), 0, s, (void*)y, (const void*)u, \
                      stride, (const void*)w, (const void*)bias, (const void*)in_bias, (const void*)state,     \
-                     (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots, C, taps)
+                     (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots, C, taps, act)
   if (f32) { if (vec) SM_CONV(float, float, 8); else SM_CONV(float, float, 1); }
   else if (out_f32) { if (vec) SM_CONV(bf16, float, 8); else SM_CONV(bf16, float, 1); }
   else { if (vec) SM_CONV(bf16, bf16, 8); else SM_CONV(bf16, bf16, 1); }
@@ -910,6 +967,76 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
   // the projection's last taps - 1 rows of every sequence become its new tail
   if (taps > 1)
     launch_conv_state(state, qkv, (long)C, cu, positions, slots, seqs, C, taps, f32, C % 8 == 0, stream);
+}
+
+// --------------------------------------------------------------------------- attention input: row norm + half-split rotation + append
+// From a fused projection row [.. | q (H D) | k (G D) | v (G Dv) | ..] (row stride ld, q at column `col0`):
+// an RMS norm over the WHOLE q projection and over the whole k projection (all heads at once, plain
+// weights qw [H D] / kw [G D]), then the half-split rotation of the first 2 nrot dimensions of every head:
+// dimension i < nrot is paired with dimension i + nrot, the pair turns by float(pos) * freqs[i].  q goes to
+// q_out [T, H, D]; k and v (unchanged) are appended at slot_mapping to caches k [NB, G, BS, D] / v [NB, G, Dv, BS].
+// One workgroup per token; norms, angles and the rotation are float32.
+template <typename T>
+__global__ void __launch_bounds__(256) sm_rownorm_rope_kernel(
+    void* __restrict__ q_out_, const void* __restrict__ qkv_, long ld, int col0, const void* __restrict__ qw_,
+    const void* __restrict__ kw_, const float* __restrict__ freqs, int nrot, float eps, void* __restrict__ k_cache_,
+    void* __restrict__ v_cache_, const int32_t* __restrict__ slot_mapping, const int32_t* __restrict__ positions, int H,
+    int G, int D, int Dv, int bs) {
+  __shared__ float red[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const T* q = (const T*)qkv_ + (size_t)t * ld + col0;
+  const T* k = q + (size_t)H * D;
+  const T* v = k + (size_t)G * D;
+  const T* qw = (const T*)qw_;
+  const T* kw = (const T*)kw_;
+  const int nq = H * D, nk = G * D, nv = G * Dv;
+  float sq = 0.f, sk = 0.f;
+  for (int e = tid; e < nq; e += 256) { const float x = ldf(q + e); sq += x * x; }
+  for (int e = tid; e < nk; e += 256) { const float x = ldf(k + e); sk += x * x; }
+  sq = block_sum(sq, red);
+  sk = block_sum(sk, red);
+  const float iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
+  const float fpos = (float)positions[t];
+  const int slot = slot_mapping[t], blk = slot / bs, off = slot - blk * bs;
+  T* q_out = (T*)q_out_ + (size_t)t * nq;
+  T* kc = (T*)k_cache_;
+  T* vc = (T*)v_cache_;
+  for (int e = tid; e < nq + nk; e += 256) {
+    const bool isq = e < nq;
+    const int ee = isq ? e : e - nq;
+    const T* src = isq ? q : k;
+    const T* w = isq ? qw : kw;
+    const float inv = isq ? iq : ik;
+    const int hd = ee / D, d = ee - hd * D;
+    float x = ldf(src + ee) * inv * ldf(w + ee);
+    if (d < 2 * nrot) {
+      const int i = d < nrot ? d : d - nrot;
+      const int pe = d < nrot ? ee + nrot : ee - nrot;          // the pair's other dimension
+      const float y = ldf(src + pe) * inv * ldf(w + pe);
+      const float ang = fpos * freqs[i];
+      const float cs = cosf(ang), sn = sinf(ang);
+      x = d < nrot ? x * cs - y * sn : x * cs + y * sn;
+    }
+    if (isq) stf(q_out + ee, x);
+    else stf(kc + (((size_t)blk * G + hd) * bs + off) * D + d, x);
+  }
+  for (int e = tid; e < nv; e += 256) {
+    const int g = e / Dv, c = e - g * Dv;
+    vc[(((size_t)blk * G + g) * Dv + c) * bs + off] = v[e];
+  }
+}
+
+void sm_rownorm_rope(uintptr_t q_out, uintptr_t qkv, long ld, int col0, uintptr_t q_norm, uintptr_t k_norm,
+                     uintptr_t freqs, int nrot, float eps, uintptr_t k_cache, uintptr_t v_cache, uintptr_t slot_mapping,
+                     uintptr_t positions, int tokens, int H, int G, int D, int Dv, int bs, int f32, uintptr_t stream) {
+  if (tokens <= 0) return;
+  DLLM_HOST_CHECK(H > 0 && G > 0 && D > 0 && Dv > 0 && bs > 0 && nrot >= 0 && 2 * nrot <= D && col0 >= 0 &&
+                      ld >= col0 + (long)H * D + (long)G * (D + Dv),
+                  "rownorm_rope sizes");
+  DLLM_HOST_CHECK(q_out && k_cache && v_cache && q_norm && k_norm && (nrot == 0 || freqs), "rownorm_rope arguments");
+  SM_DISPATCH(f32, sm_rownorm_rope_kernel, dim3(tokens), dim3(256), 0, stream, (void*)q_out, (const void*)qkv, ld, col0,
+              (const void*)q_norm, (const void*)k_norm, (const float*)freqs, nrot, eps, (void*)k_cache, (void*)v_cache,
+              (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs);
 }
 
 }  // namespace dllm

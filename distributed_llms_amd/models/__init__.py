@@ -8,6 +8,9 @@ def stage_class(arch: str):
     if arch == "gikovik":
         from .gikovik import GikovikStage
         return GikovikStage
+    if arch == "zebutar":
+        from .zebutar import ZebutarStage
+        return ZebutarStage
     if arch in ("llama", "mixtral", "gpt2"):
         from .stage import ModelStage
         return ModelStage

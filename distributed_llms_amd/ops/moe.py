@@ -217,11 +217,11 @@ def grouped_choice_ffn(x: torch.Tensor, w_router: torch.Tensor, correction: Opti
         # few tokens: the float32 router product and the selection in one launch (+ the scatter)
         logits = torch.empty(t, w_router.shape[0], dtype=torch.float32, device=dev)
         k.moe_router_groups(x.data_ptr(), w_router.data_ptr(), width, w_router.shape[0], logits.data_ptr(), cp, t, e, top,
-                            groups, keep, float(scale), topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(),
+                            groups, keep, float(scale), 0, topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(),
                             offsets.data_ptr(), sorted_tok.data_ptr(), inv.data_ptr(), f32, st)
     else:
         logits = F.linear(x.float(), w_router)                   # float32 also for bf16 activations
-        k.moe_route_groups(logits.data_ptr(), logits.shape[1], cp, t, e, top, groups, keep, float(scale),
+        k.moe_route_groups(logits.data_ptr(), logits.shape[1], cp, t, e, top, groups, keep, float(scale), 0,
                            topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
                            sorted_tok.data_ptr(), inv.data_ptr(), st)
     slots = t * top
@@ -270,4 +270,124 @@ def grouped_choice_ffn(x: torch.Tensor, w_router: torch.Tensor, correction: Opti
     out = torch.empty_like(x)
     k.moe_combine_gated(out.data_ptr(), ys.data_ptr(), topk_w.data_ptr(), inv.data_ptr(), 0 if sh is None else sh.data_ptr(),
                         logits.data_ptr() + 4 * e if has_shared else 0, logits.shape[1], t, width, top, f32, st)
+    return out
+
+
+def relu_sq_(y: torch.Tensor) -> torch.Tensor:
+    """y <- max(y, 0)^2 in place (the activation of feed-forwards of the form down(relu(up x)^2))."""
+    if not y.is_cuda:
+        return y.copy_(torch.relu(y.float()).square().to(y.dtype))
+    if not y.is_contiguous() or y.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("relu_sq_: contiguous bfloat16 or float32")
+    _ext.kernels().relu_sq(y.data_ptr(), y.numel(), 1 if y.dtype == torch.float32 else 0,
+                           torch.cuda.current_stream().cuda_stream)
+    return y
+
+
+# ------------------------------------------------------------------ biased router, softmax over the chosen logits, GLU experts
+def route_softmax_top(logits: torch.Tensor, top: int, scale: float = 1.0):
+    """Reference (PyTorch, any device): the ``top`` largest logits per row (ties: the lower index) and the
+    softmax over those logits only.  Returns (weights [T, top] float32, ids [T, top] int64)."""
+    v, ids = torch.sort(logits.float(), dim=-1, descending=True, stable=True)
+    return torch.softmax(v[:, :top], -1) * scale, ids[:, :top]
+
+
+def softmax_top_ffn(x: torch.Tensor, w_router: torch.Tensor, b_router: Optional[torch.Tensor],
+                    w_gate_up: torch.Tensor, w_down: torch.Tensor, top: int,
+                    shared_gate_up: Optional[torch.Tensor] = None, shared_down: Optional[torch.Tensor] = None,
+                    scale: float = 1.0) -> torch.Tensor:
+    """Mixture of GLU experts down_e(silu(gate_e x) * (up_e x)): router logits ``w_router x + b_router``
+    are a float32 product (``w_router`` [E, W] and ``b_router`` [E] float32), every token uses the ``top``
+    experts with the largest logits, weighted by the softmax over those logits only.  ``w_gate_up``
+    [E, 2 F, W] (gate rows, then up rows), ``w_down`` [E, W, F].  ``shared_gate_up`` [2 Fs, W] /
+    ``shared_down`` [W, Fs]: an expert of the same form that every token uses, added unweighted."""
+    e, two_f, width = w_gate_up.shape
+    f = two_f // 2
+    t = x.shape[0]
+    if w_router.shape != (e, width) or w_router.dtype != torch.float32 or (
+            b_router is not None and (b_router.dtype != torch.float32 or b_router.numel() != e)):
+        raise ValueError("softmax_top_ffn: router [E, W] and bias [E] in float32")
+    if not 1 <= top <= min(e, 16):
+        raise ValueError("softmax_top_ffn: 1 <= top <= min(experts, 16)")
+    if not x.is_cuda:
+        xf = x.float()
+        tw, ids = route_softmax_top(F.linear(xf, w_router, b_router), top, scale)
+        out = torch.zeros(t, width, dtype=torch.float32)
+
+        def glu(h, wgu, wd):
+            gu = F.linear(h, wgu.float())
+            return F.linear(F.silu(gu[:, :wgu.shape[0] // 2]) * gu[:, wgu.shape[0] // 2:], wd.float())
+        for j in range(e):
+            rows, col = (ids == j).nonzero(as_tuple=True)
+            if rows.numel():
+                out.index_add_(0, rows, glu(xf[rows], w_gate_up[j], w_down[j]) * tw[rows, col, None])
+        if shared_gate_up is not None:
+            out += glu(xf, shared_gate_up, shared_down)
+        return out.to(x.dtype)
+    from . import linear
+    from .latent import linear_swiglu
+    k = _ext.kernels()
+    st = torch.cuda.current_stream().cuda_stream
+    dev = x.device
+    f32 = 1 if x.dtype == torch.float32 else 0
+    if not (x.is_contiguous() and w_gate_up.is_contiguous() and w_down.is_contiguous() and w_router.is_contiguous()):
+        raise ValueError("softmax_top_ffn: operands must be contiguous")
+    topk_w = torch.empty(t, top, dtype=torch.float32, device=dev)
+    topk_ids = torch.empty(t, top, dtype=torch.int32, device=dev)
+    counts = torch.empty(e, dtype=torch.int32, device=dev)
+    offsets = torch.empty(e + 1, dtype=torch.int32, device=dev)
+    sorted_tok = torch.empty(t * top, dtype=torch.int32, device=dev)
+    inv = torch.empty(t * top, dtype=torch.int32, device=dev)
+    bp = 0 if b_router is None else b_router.data_ptr()
+    if t <= ROUTER_FUSED_MAX_TOKENS:
+        # few tokens: the float32 router product and the selection in one launch (+ the scatter)
+        logits = torch.empty(t, e, dtype=torch.float32, device=dev)
+        k.moe_router_groups(x.data_ptr(), w_router.data_ptr(), width, e, logits.data_ptr(), bp, t, e, top, 1, 1,
+                            float(scale), 1, topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(),
+                            offsets.data_ptr(), sorted_tok.data_ptr(), inv.data_ptr(), f32, st)
+    else:
+        logits = F.linear(x.float(), w_router)                   # float32 also for bf16 activations
+        k.moe_route_groups(logits.data_ptr(), e, bp, t, e, top, 1, 1, float(scale), 1, topk_w.data_ptr(),
+                           topk_ids.data_ptr(), counts.data_ptr(), offsets.data_ptr(), sorted_tok.data_ptr(),
+                           inv.data_ptr(), st)
+    slots = t * top
+    ys = torch.empty(slots, width, dtype=x.dtype, device=dev)
+    bf = x.dtype == torch.bfloat16
+    cp, op = counts.data_ptr(), offsets.data_ptr()
+    if bf and t <= GROUPED_MAX_TOKENS and width % 128 == 0 and f % 128 == 0:
+        # decode-sized: grouped GEMMs on the expert-sorted slots with the SwiGLU in the first one's
+        # epilogue, no host sync (the MFMA-tiled kernel from several rows per expert on)
+        act = torch.empty(slots, f, dtype=x.dtype, device=dev)
+        if 0 < knobs.K.moe_wide_min_pairs <= slots:
+            ring = 0 if knobs.K.moe_deep_ring else 4
+            k.moe_wide_gemm(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_gate_up.data_ptr(), cp, op, e, two_f,
+                            width, 1 | ring, st)
+            k.moe_wide_gemm(ys.data_ptr(), act.data_ptr(), 0, w_down.data_ptr(), cp, op, e, width, f, ring, st)
+        else:
+            rows = -(-slots // e)
+            k.moe_grouped_gemm(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_gate_up.data_ptr(), cp, op, e,
+                               two_f, width, 1, rows, knobs.K.moe_variant, st)
+            k.moe_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, w_down.data_ptr(), cp, op, e, width, f, 0, rows,
+                               knobs.K.moe_variant, st)
+    elif bf and two_f % 256 == 0 and width % 256 == 0 and f % 64 == 0 and t * width * 2 < (1 << 32) \
+            and slots * f * 2 < (1 << 32):
+        # prompt-sized: one grouped 256 x 256-tile launch per projection over every expert's row tiles
+        act = torch.empty(slots, f, dtype=x.dtype, device=dev)
+        k.gemm_pp_moe(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_gate_up.data_ptr(), cp, op, e, two_f,
+                      width, t, slots, 1, st)
+        k.gemm_pp_moe(ys.data_ptr(), act.data_ptr(), 0, w_down.data_ptr(), cp, op, e, width, f, slots, slots, 0, st)
+    else:
+        # float32 and odd expert sizes: per-expert library GEMMs, counts read on the host
+        xs = x.index_select(0, sorted_tok.long())
+        off = offsets.cpu().tolist()
+        for j in range(e):
+            a, b = off[j], off[j + 1]
+            if b > a:
+                ys[a:b] = F.linear(linear_swiglu(xs[a:b], w_gate_up[j]), w_down[j])
+    sh = None
+    if shared_gate_up is not None:
+        sh = linear(linear_swiglu(x, shared_gate_up), shared_down)
+    out = torch.empty_like(x)
+    k.moe_combine_gated(out.data_ptr(), ys.data_ptr(), topk_w.data_ptr(), inv.data_ptr(), 0 if sh is None else sh.data_ptr(),
+                        0, 0, t, width, top, f32, st)
     return out

@@ -79,6 +79,25 @@ def embedding_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def embedding_norm_f32(ids: torch.Tensor, table: torch.Tensor, w: torch.Tensor, eps: float, one_plus: bool = True,
+                       rounded: bool = False):
+    """The RMS norm of the looked-up rows, rms(table[ids]) * ((1 if one_plus else 0) + w), as a float32
+    residual stream [T, W]; with ``rounded`` also in the table's dtype (the stream tensor itself when that
+    is float32): the input of a first sublayer that reads the stream unnormed."""
+    if not table.is_cuda:
+        x = _ref_rms(table.index_select(0, ids.long()), w, eps, 1.0 if one_plus else 0.0)
+        return x, ((x if table.dtype == torch.float32 else x.to(table.dtype)) if rounded else None)
+    _ck(ids, "ids", torch.int32)
+    _ck(table, "table")
+    _ck(w, "w", table.dtype)
+    t, (v, width) = ids.numel(), table.shape
+    x = torch.empty(t, width, dtype=torch.float32, device=table.device)
+    h = torch.empty(t, width, dtype=table.dtype, device=table.device) if rounded and table.dtype != torch.float32 else None
+    _k().sm_embed_norm(x.data_ptr(), _ptr(h), ids.data_ptr(), table.data_ptr(), w.data_ptr(), t, width, v, float(eps),
+                       1.0 if one_plus else 0.0, _f32flag(table), _stream())
+    return x, ((x if h is None else h) if rounded else None)
+
+
 def _ref_rms(x: torch.Tensor, w: torch.Tensor, eps: float, offset: float) -> torch.Tensor:
     x = x.float()
     return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
@@ -98,25 +117,35 @@ def rms_norm_f32(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype, one_pl
 
 
 def post_norm_add(x: torch.Tensor, o: torch.Tensor, w_post: torch.Tensor, eps: float, mult: float,
-                  bias: Optional[torch.Tensor] = None, w_next: Optional[torch.Tensor] = None, one_plus: bool = True):
+                  bias: Optional[torch.Tensor] = None, w_next: Optional[torch.Tensor] = None, one_plus: bool = True,
+                  o2: Optional[torch.Tensor] = None, scales=(1.0, 1.0), plain_next: bool = False):
     """The close of a sublayer, fused: ``x += mult * rms_norm(o + bias) * (1 + w_post)`` in place on the
     float32 residual stream; with ``w_next`` also returns the next sublayer's input
     ``rms_norm(x) * (1 + w_next)`` in ``o``'s dtype (None otherwise).  ``one_plus`` False: both norm
-    weights are plain (``* w``)."""
+    weights are plain (``* w``).  ``o2``: the sublayer's output is ``scales[0] * o + scales[1] * o2`` (two
+    mixers side by side).  ``plain_next`` (without ``w_next``): the next sublayer reads the stream itself;
+    returns it in ``o``'s dtype (the stream tensor when that is float32)."""
     off = 1.0 if one_plus else 0.0
     if not x.is_cuda:
-        ob = o.float() if bias is None else o.float() + bias.float()
+        ob = o.float() if o2 is None else scales[0] * o.float() + scales[1] * o2.float()
+        if bias is not None:
+            ob = ob + bias.float()
         x.add_(mult * _ref_rms(ob, w_post, eps, off))
-        return x, (None if w_next is None else _ref_rms(x, w_next, eps, off).to(o.dtype))
+        if w_next is None:
+            return x, ((x if o.dtype == torch.float32 else x.to(o.dtype)) if plain_next else None)
+        return x, _ref_rms(x, w_next, eps, off).to(o.dtype)
     _ck(x, "x", torch.float32)
     _ck(o, "o")
     t, width = x.shape
-    if o.shape != x.shape:
+    if o.shape != x.shape or (o2 is not None and (o2.shape != x.shape or o2.dtype != o.dtype or not o2.is_contiguous())):
         raise ValueError("post_norm_add: o / x shape mismatch")
-    h = torch.empty_like(o) if w_next is not None else None
+    h = None
+    if w_next is not None or (plain_next and o.dtype != torch.float32):
+        h = torch.empty_like(o)
     _k().sm_post_norm_add(x.data_ptr(), o.data_ptr(), _ptr(bias), w_post.data_ptr(), _ptr(w_next), _ptr(h), t, width,
-                          float(eps), float(mult), off, _f32flag(o), _stream())
-    return x, h
+                          float(eps), float(mult), off, _ptr(o2), float(scales[0]), float(scales[1]), _f32flag(o),
+                          _stream())
+    return x, (x if (plain_next and w_next is None and h is None) else h)
 
 
 # ------------------------------------------------------------------ causal convolution with state
@@ -148,11 +177,15 @@ def _ref_conv_gather(u: torch.Tensor, state: torch.Tensor, sb: SeqBatch, taps: i
 
 
 def causal_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
-                sb: SeqBatch, out_dtype=torch.float32, in_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                sb: SeqBatch, out_dtype=torch.float32, in_bias: Optional[torch.Tensor] = None,
+                act: Optional[str] = None) -> torch.Tensor:
     """Per-channel causal convolution over time, y_t = bias + sum_j w[:, j] (u + in_bias)_(t - taps + 1 + j)
     (zeros before the sequence's start), across chunk borders: ``state`` [slots, taps - 1, C] holds each
     sequence's last taps - 1 rows of ``u`` and is brought up to date.  ``u`` [T, C] may be a column slice
-    of a wider projection (row stride); ``in_bias`` is the bias of the projection that made it."""
+    of a wider projection (row stride); ``in_bias`` is the bias of the projection that made it.  ``w`` is
+    tap-major [taps, C], the last row the current token's.  ``act`` "silu": y <- y sigmoid(y) (float32)."""
+    if act not in (None, "silu"):
+        raise ValueError(f"causal_conv: activation {act!r} (None, 'silu')")
     taps, c = w.shape
     if u.shape[1] != c or state.shape[1:] != (taps - 1, c):
         raise ValueError("causal_conv: shape mismatch")
@@ -161,6 +194,8 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
         y = (g * w.float()[:, None, :]).sum(0)
         if bias is not None:
             y = y + bias.float()
+        if act == "silu":
+            y = y * torch.sigmoid(y)
         return y.to(out_dtype)
     if u.stride(1) != 1:
         raise ValueError("causal_conv: channels must be contiguous")
@@ -170,7 +205,7 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _k().sm_causal_conv(y.data_ptr(), u.data_ptr(), u.stride(0), w.data_ptr(), _ptr(bias), _ptr(in_bias), state.data_ptr(),
                         sb.cu.data_ptr(), sb.positions.data_ptr(), sb.tok_seq.data_ptr(), sb.state_slots.data_ptr(),
                         sb.num_tokens, sb.num_seqs, c, taps, _f32flag(u), 1 if out_dtype == torch.float32 else 0,
-                        _stream())
+                        1 if act == "silu" else 0, _stream())
     return y
 
 
@@ -357,6 +392,64 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
     return q
 
 
+# ------------------------------------------------------------------ attention input: row norm + half-split rotation + append
+def rotary_frequencies(dims: int, base: float) -> torch.Tensor:
+    """f_i = base^(-2i / dims), i < dims / 2, computed in float64 and rounded once to float32."""
+    return yarn_frequencies(dims, base, None)[0]
+
+
+def _ref_rope_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+    """x [T, H, D] float32; dimension i < len(freqs) is paired with dimension i + len(freqs); the pair
+    (u, v) turns to (u cos a - v sin a, v cos a + u sin a), a = pos * f_i."""
+    n = freqs.numel()
+    ang = pos.float()[:, None] * freqs.float()[None]
+    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    out = x.clone()
+    a, b = x[..., :n], x[..., n:2 * n]
+    out[..., :n] = a * c - b * s
+    out[..., n:2 * n] = b * c + a * s
+    return out
+
+
+def rownorm_rope(qkv: torch.Tensor, col0: int, q_norm: torch.Tensor, k_norm: torch.Tensor, freqs: torch.Tensor,
+                 eps: float, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                 positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """From columns ``col0 ..`` of a fused projection [T, .. | q (heads dim) | k (kv_heads dim) | v (kv_heads
+    vdim) | ..]: an RMS norm over the WHOLE q projection and over the whole k projection (all heads at
+    once; plain weights ``q_norm`` [heads dim], ``k_norm`` [kv_heads dim]), then the half-split rotation
+    of the first 2 len(freqs) dimensions of every q and k head (dimension i paired with i + len(freqs),
+    angle position * freqs[i]), and the append of k and v (v unchanged) at ``slot_mapping`` into caches
+    k [NB, kv_heads, BS, dim] / v [NB, kv_heads, vdim, BS].  Returns q [T, heads, dim]."""
+    t = qkv.shape[0]
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    if qkv.shape[1] < col0 + nq + nk + nv or q_norm.numel() != nq or k_norm.numel() != nk or 2 * freqs.numel() > dim:
+        raise ValueError("rownorm_rope: shape mismatch")
+    bs = k_cache.shape[2]
+    if k_cache.shape[1:] != (kv_heads, bs, dim) or v_cache.shape[1:] != (kv_heads, vdim, bs):
+        raise ValueError("rownorm_rope: cache shape")
+    if not qkv.is_cuda:
+        x = qkv[:, col0:col0 + nq + nk + nv].float()
+        q = _ref_rope_half(_ref_rms(x[:, :nq], q_norm, eps, 0.0).view(t, heads, dim), positions, freqs)
+        k = _ref_rope_half(_ref_rms(x[:, nq:nq + nk], k_norm, eps, 0.0).view(t, kv_heads, dim), positions, freqs)
+        slot = slot_mapping.long()
+        k_cache[slot // bs, :, slot % bs] = k.to(k_cache.dtype)
+        v_cache[slot // bs, :, :, slot % bs] = qkv[:, col0 + nq + nk:col0 + nq + nk + nv].reshape(t, kv_heads, vdim).to(
+            v_cache.dtype)
+        return q.to(qkv.dtype)
+    _ck(qkv, "qkv")
+    _ck(q_norm, "q_norm", qkv.dtype)
+    _ck(k_norm, "k_norm", qkv.dtype)
+    _ck(freqs, "freqs", torch.float32)
+    _ck(k_cache, "k_cache", qkv.dtype)
+    _ck(v_cache, "v_cache", qkv.dtype)
+    q = torch.empty(t, heads, dim, dtype=qkv.dtype, device=qkv.device)
+    _k().sm_rownorm_rope(q.data_ptr(), qkv.data_ptr(), qkv.shape[1], int(col0), q_norm.data_ptr(), k_norm.data_ptr(),
+                         freqs.data_ptr(), freqs.numel(), float(eps), k_cache.data_ptr(), v_cache.data_ptr(),
+                         slot_mapping.data_ptr(), positions.data_ptr(), t, heads, kv_heads, dim, vdim, bs,
+                         _f32flag(qkv), _stream())
+    return q
+
+
 # ------------------------------------------------------------------ sliding-window attention
 DECODE_SPLIT_KEYS = 256     # fewest keys worth a workgroup of their own
 DECODE_TARGET_WGS = 512     # workgroups wanted on the chip (256 CUs, two each)
@@ -371,9 +464,11 @@ def decode_splits(rows: int, heads: int, kv_heads: int, ctx: int) -> int:
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                      sb: SeqBatch, window: int, scale: float, num_decode: Optional[int] = None,
-                     sinks: Optional[torch.Tensor] = None, max_ctx: Optional[int] = None) -> torch.Tensor:
+                     sinks: Optional[torch.Tensor] = None, max_ctx: Optional[int] = None, chunk: int = 0) -> torch.Tensor:
     """Softmax attention of every query token over the keys j of its own sequence with
-    0 <= p - j < window (p the query's position), keys / values read through ``block_tables`` from
+    0 <= p - j < window (p the query's position) and, with ``chunk`` > 0, floor(j / chunk) =
+    floor(p / chunk) (attention inside fixed chunks of positions counted from position 0, wherever a
+    prompt was cut for processing), keys / values read through ``block_tables`` from
     caches k [NB, G, BS, dim] / v [NB, G, vdim, BS]; query head h reads K/V head h // (H / G).
     Scores and weights are float32.  ``num_decode``: the first that many sequences are one-token
     rows (they take the decode kernel; None: every sequence is one); the rest are prompt chunks.
@@ -390,7 +485,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         rep = h // g
         for i in range(t):
             p = pos[i]
-            lo = max(0, p - window + 1)
+            lo = max(0, p - window + 1, p - p % chunk if chunk > 0 else 0)
             idx = torch.arange(lo, p + 1)
             blk = block_tables[seq[i]].long()[idx // bs]
             kk = k_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)     # [n, H, d]
@@ -406,7 +501,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _ck(k_cache, "k_cache", q.dtype)
     _ck(v_cache, "v_cache", q.dtype)
     _ck(block_tables, "block_tables", torch.int32)
-    if h % g or k_cache.shape[3] != d or v_cache.shape[3] != bs or window < 1:
+    if h % g or k_cache.shape[3] != d or v_cache.shape[3] != bs or window < 1 or chunk < 0:
         raise ValueError("window_attention: head / size mismatch")
     if sinks is not None:
         _ck(sinks, "sinks", torch.float32)
@@ -416,17 +511,18 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     nd = sb.num_seqs if num_decode is None else int(num_decode)
     f = _f32flag(q)
     if nd:       # one-token rows are the first nd tokens
-        splits, ws = decode_splits(nd, h, g, min(int(window), int(max_ctx or 0))), None
+        span = min(int(window), int(chunk)) if chunk > 0 else int(window)
+        splits, ws = decode_splits(nd, h, g, min(span, int(max_ctx or 0))), None
         if splits > 1 and not f:
             ws = torch.empty(nd * h * splits * (dv + 2), dtype=torch.float32, device=q.device)
         _k().sm_window_attn_decode(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                    block_tables.data_ptr(), block_tables.shape[1], sb.positions.data_ptr(),
-                                   sb.tok_seq.data_ptr(), nd, h, g, d, dv, bs, int(window), float(scale), _ptr(sinks),
+                                   sb.tok_seq.data_ptr(), nd, h, g, d, dv, bs, int(window), int(chunk), float(scale), _ptr(sinks),
                                    splits if ws is not None else 1, _ptr(ws), f, _stream())
     if t > nd:
         _k().sm_window_attn_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                     block_tables.data_ptr(), block_tables.shape[1], sb.cu.data_ptr(),
                                     sb.positions.data_ptr(), sb.tok_seq.data_ptr(), nd, sb.num_seqs, t, sb.max_q_len,
                                     h, g, d, dv, bs,
-                                    int(window), float(scale), _ptr(sinks), f, _stream())
+                                    int(window), int(chunk), float(scale), _ptr(sinks), f, _stream())
     return out
