@@ -159,11 +159,17 @@ def route_top(z, top):
     return idx, e / e.sum()
 
 
-def moe_ff(h, w, mlp):
+def moe_ff(h, w, mlp, margins=None):
+    """``margins``: a list that receives, per token, the gap between the last chosen logit and the best
+    one left out (how far the choice is from turning over)."""
     out = np.zeros_like(h)
     z = h @ w["router"].T + w["router.b"]
+    top = mlp["router"]["top"]
+    if margins is not None:
+        zs = -np.sort(-z, axis=-1)
+        margins.append(zs[:, top - 1] - zs[:, top] if top < z.shape[1] else np.full(h.shape[0], np.inf))
     for i in range(h.shape[0]):
-        idx, p = route_top(z[i], mlp["router"]["top"])
+        idx, p = route_top(z[i], top)
         for j, pj in zip(idx, p):
             out[i] += pj * glu_expert(h[i:i + 1], sub(w, f"e{j}."))[0]
     if mlp.get("shared"):
@@ -171,9 +177,74 @@ def moe_ff(h, w, mlp):
     return out
 
 
-def forward(cfg, sd, tokens, taps=None):
+def shapes(cfg):
+    """Checkpoint name -> shape."""
+    w = cfg["width"]
+    s = {"embed": (cfg["vocab"], w), "embed.norm": (w,), "final.norm": (w,), "head": (cfg["vocab"], w)}
+    for i, layer in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        l, r = layer["mixer"]["left"], layer["mixer"]["right"]
+        s[p + "norm1"] = (w,)
+        s.update({p + "mix.left.q": (l["heads"] * l["dim"], w), p + "mix.left.k": (l["kv_heads"] * l["dim"], w),
+                  p + "mix.left.v": (l["kv_heads"] * l["vdim"], w), p + "mix.left.q.norm": (l["heads"] * l["dim"],),
+                  p + "mix.left.k.norm": (l["kv_heads"] * l["dim"],), p + "mix.left.o": (w, l["heads"] * l["vdim"])})
+        qk, vv = r["kv_heads"] * r["dim"], r["heads"] * r["vdim"]
+        s.update({p + "mix.right.q": (qk, w), p + "mix.right.q.conv": (qk, r["conv"]), p + "mix.right.k": (qk, w),
+                  p + "mix.right.k.conv": (qk, r["conv"]), p + "mix.right.v": (vv, w),
+                  p + "mix.right.v.conv": (vv, r["conv"]), p + "mix.right.b": (r["heads"], w),
+                  p + "mix.right.a": (r["heads"], w), p + "mix.right.A_log": (r["heads"],),
+                  p + "mix.right.dt_bias": (r["heads"],), p + "mix.right.g": (vv, w), p + "mix.right.norm": (r["vdim"],),
+                  p + "mix.right.o": (w, vv)})
+        mlp = layer.get("mlp")
+        if not mlp:
+            continue
+        s[p + "norm2"] = (w,)
+        if mlp["kind"] == "dense":
+            s.update({p + "mlp.up": (mlp["ff"], w), p + "mlp.down": (w, mlp["ff"])})
+        else:
+            f = mlp["expert"]["ff"]
+            s.update({p + "mlp.router": (mlp["router"]["experts"], w), p + "mlp.router.b": (mlp["router"]["experts"],)})
+            for j in range(mlp["router"]["experts"]):
+                s.update({p + f"mlp.e{j}.gate": (f, w), p + f"mlp.e{j}.up": (f, w), p + f"mlp.e{j}.down": (w, f)})
+            if mlp.get("shared"):
+                fs = mlp["shared"]["ff"]
+                s.update({p + "mlp.shared.gate": (fs, w), p + "mlp.shared.up": (fs, w), p + "mlp.shared.down": (w, fs)})
+    return s
+
+
+def make_weights(cfg, seed=0):
+    """Random float64 weights under the checkpoint names: projections ~ N(0, 1 / fan_in), stream norms
+    stored around zero, plain norms around one, decays from slow to fast per head, a router wide enough
+    that few choices are close calls."""
+    rng = np.random.default_rng(seed)
+    sd = {}
+    for name, shape in shapes(cfg).items():
+        leaf = name.rsplit(".", 1)[-1]
+        if leaf in ("norm1", "norm2") or name in ("embed.norm", "final.norm"):
+            t = 0.15 * rng.standard_normal(shape)
+        elif leaf == "norm":
+            t = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif leaf == "A_log":
+            t = rng.uniform(-4.0, 0.5, shape)
+        elif leaf == "dt_bias":
+            t = rng.standard_normal(shape)
+        elif leaf == "conv":
+            t = rng.standard_normal(shape) / shape[1] ** 0.5
+        elif name.endswith("router.b"):
+            t = 0.5 * rng.standard_normal(shape)
+        elif leaf == "router":
+            t = 4.0 * rng.standard_normal(shape) / shape[-1] ** 0.5
+        elif name == "embed":
+            t = rng.standard_normal(shape)
+        else:
+            t = rng.standard_normal(shape) / shape[-1] ** 0.5
+        sd[name] = t
+    return sd
+
+
+def forward(cfg, sd, tokens, taps=None, margins=None):
     """Logits [T, vocab] of one whole sequence.  ``sd``: checkpoint name -> float64 array.  ``taps``: a
-    list that receives the stream after every layer."""
+    list that receives the stream after every layer; ``margins``: one that receives every router's."""
     eps = cfg["norm"]["eps"]
     x = norm_one_plus(sd["embed"][np.asarray(tokens)], sd["embed.norm"], eps)
     for i, layer in enumerate(cfg["layers"]):
@@ -183,7 +254,7 @@ def forward(cfg, sd, tokens, taps=None):
         x = x + norm_one_plus(parallel_mixer(x, sub(w, "mix."), layer["mixer"], eps), w["norm1"], eps)
         mlp = layer.get("mlp")
         if mlp:
-            f = dense_ff(x, sub(w, "mlp.")) if mlp["kind"] == "dense" else moe_ff(x, sub(w, "mlp."), mlp)
+            f = dense_ff(x, sub(w, "mlp.")) if mlp["kind"] == "dense" else moe_ff(x, sub(w, "mlp."), mlp, margins)
             x = x + norm_one_plus(f, w["norm2"], eps)
         if taps is not None:
             taps.append(x.copy())
