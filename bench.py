@@ -90,7 +90,9 @@ def parse(argv=None):
                          "prompts of --prompt-len tokens then --gen-len decode steps; one JSON line per size")
     ap.add_argument("--hybrid-models", default="tudilix,llama",
                     help="--hybrid: the models to run: tudilix,llama (sliding-window attention + RG-LRU beside Llama) "
-                         "or gikovik,mixtral (latent attention + grouped-choice experts beside Mixtral), or one of them")
+                         "or gikovik,mixtral (latent attention + grouped-choice experts beside Mixtral), or "
+                         "zebutar,mixtral (chunked attention beside a gated delta rule + SwiGLU experts beside "
+                         "Mixtral), or one of them")
     return ap.parse_args(argv)
 
 

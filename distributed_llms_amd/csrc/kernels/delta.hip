@@ -9,7 +9,8 @@
 //                       sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias))
 //   dr_scan_kernel      the recurrence over a varlen batch: a workgroup per (sequence, head, 64 value
 //                       columns); a column's state is thread-local (split over 4 lanes along dim), so a
-//                       step costs no exchange besides two 4-lane sums
+//                       step costs no exchange besides two 4-lane sums; optionally with dr_prep_kernel's
+//                       work done on the staged tokens (the product path)
 //   dr_out_norm_kernel  per (token, head): o / rms(o) * w * silu(gate)
 #include <math.h>
 
@@ -59,97 +60,187 @@ void dr_prep(uintptr_t u, long ld, uintptr_t ab, long ldab, int bcol, uintptr_t 
 // The recurrence.  Lane (part = lane / 16, jj = lane % 16) of wave w owns rows [part DK/4, (part + 1) DK/4) of
 // value column j = 64 z + 16 w + jj of the state of head h: S^T k and S^T q are DK/4 FMAs and a sum over the
 // four parts.  k and q (zero-padded to DK) and the gates of kDrTB tokens are staged in LDS for the
-// workgroup's four waves.  A chunk that starts at position 0 starts from a zero state; the state goes
-// back to its slot after the chunk's last token.
+// workgroup's four waves; the next block's global loads are issued before the current block's steps and
+// land in LDS after them.  With `ab_` the kernel takes the RAW q and k (after convolution and activation)
+// and the gate logits and does dr_prep_kernel's work on the staged block itself (unit norms, beta, g), so
+// the mixer needs no pass of its own for them.  A chunk that starts at position 0 starts from a zero
+// state; the state goes back to its slot after the chunk's last token.
 constexpr int kDrTB = 8;
 
-template <int DK>
+template <int DK, int CPL, typename T>
 __global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, const float* __restrict__ u, long ld,
-                                                      const float* __restrict__ bd, float* __restrict__ state,
-                                                      const int32_t* __restrict__ cu,
+                                                      const float* __restrict__ bd, const void* __restrict__ ab_,
+                                                      long ldab, int bcol, const float* __restrict__ a_log,
+                                                      const float* __restrict__ dt_bias, float qscale, float unit_eps,
+                                                      float* __restrict__ state, const int32_t* __restrict__ cu,
                                                       const int32_t* __restrict__ positions,
                                                       const int32_t* __restrict__ slots, int H, int G, int dim,
                                                       int vdim) {
   constexpr int R = DK / 4;
+  constexpr int NST = kDrTB * 2 * DK / 256;                   // staged k / q elements per thread and block
   __shared__ __attribute__((aligned(16))) float kq[kDrTB][2][DK];
   __shared__ float gates[kDrTB][2];
   const int b = blockIdx.x, h = blockIdx.y;
   const int lo = cu[b], n = cu[b + 1] - lo;
   if (n <= 0) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, part = lane >> 4, jj = lane & 15;
-  const int j = blockIdx.z * 64 + wave * 16 + jj;
-  const bool jok = j < vdim;
+  // CPL value columns per lane, 64 apart: every k / q element a lane reads from LDS feeds CPL columns (the
+  // LDS reads, not the FMAs, bound the CPL = 1 form on long chunks)
+  int j[CPL];
+  bool jok[CPL];
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) {
+    j[c] = (blockIdx.z * CPL + c) * 64 + wave * 16 + jj;
+    jok[c] = j[c] < vdim;
+  }
   const int g = h / (H / G);
   const size_t kcol = (size_t)G * dim + (size_t)g * dim, qcol = (size_t)g * dim, vcol = 2 * (size_t)G * dim + (size_t)h * vdim;
+  const T* ab = (const T*)ab_;
+  const float ea = ab ? expf(a_log[h]) : 0.f, dtb = ab ? dt_bias[h] : 0.f;
   float* S = state + ((size_t)slots[b] * H + h) * dim * vdim;
   const bool fresh = positions[lo] == 0;
-  float s[R];
+  float s[CPL][R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = part * R + r;
-    s[r] = (!fresh && jok && i < dim) ? S[(size_t)i * vdim + j] : 0.f;
-  }
+  for (int c = 0; c < CPL; ++c)
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int i = part * R + r;
+      s[c][r] = (!fresh && jok[c] && i < dim) ? S[(size_t)i * vdim + j[c]] : 0.f;
+    }
+  float st[NST], vn[CPL][kDrTB], gn = 0.f;
+  auto fetch = [&](int t0) {                                  // global loads of the block that starts at t0
+    const int nt = min(kDrTB, n - t0);
+#pragma unroll
+    for (int r = 0; r < NST; ++r) {
+      const int idx = tid + 256 * r;
+      const int tt = idx / (2 * DK), rem = idx - tt * 2 * DK, which = rem / DK, i = rem - which * DK;
+      st[r] = (tt < nt && i < dim) ? u[(size_t)(lo + t0 + tt) * ld + (which ? qcol : kcol) + i] : 0.f;
+    }
+#pragma unroll
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+      for (int tt = 0; tt < kDrTB; ++tt)
+        vn[c][tt] = (tt < nt && jok[c]) ? u[(size_t)(lo + t0 + tt) * ld + vcol + j[c]] : 0.f;
+    if (tid < nt * 2) {
+      const int tt = tid >> 1, w = tid & 1;
+      gn = ab ? ldf(ab + (size_t)(lo + t0 + tt) * ldab + bcol + w * H + h)
+              : bd[(size_t)(lo + t0 + tt) * 2 * H + w * H + h];
+    }
+  };
+  fetch(0);
   for (int t0 = 0; t0 < n; t0 += kDrTB) {
     const int nt = min(kDrTB, n - t0);
     __syncthreads();                                          // the previous block's reads are done
-    for (int idx = tid; idx < nt * 2 * DK; idx += 256) {
-      const int tt = idx / (2 * DK), rem = idx - tt * 2 * DK, which = rem / DK, i = rem - which * DK;
-      const float* row = u + (size_t)(lo + t0 + tt) * ld;
-      kq[tt][which][i] = i < dim ? row[(which ? qcol : kcol) + i] : 0.f;
-    }
-    if (tid < nt * 2) gates[tid >> 1][tid & 1] = bd[(size_t)(lo + t0 + (tid >> 1)) * 2 * H + (tid & 1) * H + h];
-    float vv[kDrTB];
 #pragma unroll
-    for (int tt = 0; tt < kDrTB; ++tt) vv[tt] = (tt < nt && jok) ? u[(size_t)(lo + t0 + tt) * ld + vcol + j] : 0.f;
+    for (int r = 0; r < NST; ++r) {
+      const int idx = tid + 256 * r;
+      (&kq[0][0][0])[idx] = st[r];
+    }
+    if (tid < nt * 2) {
+      float gv = gn;
+      if (ab) gv = (tid & 1) ? expf(-ea * dr_softplus(gn + dtb)) : dr_sigmoid(gn);
+      gates[tid >> 1][tid & 1] = gv;
+    }
+    float vv[CPL][kDrTB];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+      for (int tt = 0; tt < kDrTB; ++tt) vv[c][tt] = vn[c][tt];
+    if (ab) {                                                 // unit norms of the staged k and q vectors
+      __syncthreads();
+      for (int vec = wave; vec < nt * 2; vec += 4) {
+        float* x = &kq[0][0][0] + vec * DK;
+        float ss = 0.f;
+        for (int i = lane; i < DK; i += 64) ss += x[i] * x[i];
+        ss = wave_sum(ss);
+        const float m = ((vec & 1) ? qscale : 1.0f) / sqrtf(ss + unit_eps);
+        for (int i = lane; i < DK; i += 64) x[i] *= m;
+      }
+    }
     __syncthreads();
+    if (t0 + kDrTB < n) fetch(t0 + kDrTB);
 #pragma unroll
     for (int tt = 0; tt < kDrTB; ++tt) {
       if (tt < nt) {
         const float* kk = &kq[tt][0][part * R];
         const float* qq = &kq[tt][1][part * R];
         const float beta = gates[tt][0], dec = gates[tt][1];
-        float acc = 0.f;
+        float a4[CPL][4], o4[CPL][4], uj[CPL];
+#pragma unroll
+        for (int c = 0; c < CPL; ++c)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a4[c][e] = o4[c][e] = 0.f;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          s[r] *= dec;
-          acc = fmaf(s[r], kk[r], acc);
+          const float kr = kk[r];
+#pragma unroll
+          for (int c = 0; c < CPL; ++c) {
+            s[c][r] *= dec;
+            a4[c][r & 3] = fmaf(s[c][r], kr, a4[c][r & 3]);
+          }
         }
-        acc = rows_sum(acc);
-        const float uj = beta * (vv[tt] - acc);
-        float oo = 0.f;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c)
+          uj[c] = beta * (vv[c][tt] - rows_sum((a4[c][0] + a4[c][1]) + (a4[c][2] + a4[c][3])));
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          s[r] = fmaf(kk[r], uj, s[r]);
-          oo = fmaf(s[r], qq[r], oo);
+          const float kr = kk[r], qr = qq[r];
+#pragma unroll
+          for (int c = 0; c < CPL; ++c) {
+            s[c][r] = fmaf(kr, uj[c], s[c][r]);
+            o4[c][r & 3] = fmaf(s[c][r], qr, o4[c][r & 3]);
+          }
         }
-        oo = rows_sum(oo);
-        if (part == 0 && jok) o[((size_t)(lo + t0 + tt) * H + h) * vdim + j] = oo;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+          const float oo = rows_sum((o4[c][0] + o4[c][1]) + (o4[c][2] + o4[c][3]));
+          if (part == 0 && jok[c]) o[((size_t)(lo + t0 + tt) * H + h) * vdim + j[c]] = oo;
+        }
       }
     }
   }
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = part * R + r;
-    if (jok && i < dim) S[(size_t)i * vdim + j] = s[r];
-  }
+  for (int c = 0; c < CPL; ++c)
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int i = part * R + r;
+      if (jok[c] && i < dim) S[(size_t)i * vdim + j[c]] = s[c][r];
+    }
 }
 
-void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t state, uintptr_t cu, uintptr_t positions,
-             uintptr_t slots, int seqs, int H, int G, int dim, int vdim, uintptr_t stream) {
+// `bd` [T, 2 H] (beta | g) with unit q and k in `u`, or -- bd null -- `ab` [T, ldab] in the activation type (f32:
+// float) holding the raw logits b | a from column `bcol`, with raw q and k in `u`.
+void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long ldab, int bcol, uintptr_t a_log,
+             uintptr_t dt_bias, float qscale, float unit_eps, uintptr_t state, uintptr_t cu, uintptr_t positions,
+             uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, int f32, uintptr_t stream) {
   if (seqs <= 0) return;
   DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && dim > 0 && dim <= 256 && vdim > 0 && H <= 65535 &&
                       ld >= 2L * G * dim + (long)H * vdim,
                   "delta rule sizes (key size up to 256)");
-  const dim3 grid(seqs, H, (vdim + 63) / 64);
+  DLLM_HOST_CHECK((bd != 0) != (ab != 0) && (!ab || (a_log && dt_bias && ldab >= bcol + 2L * H && bcol >= 0)),
+                  "delta rule gates: beta | g, or the raw logits with A_log and dt_bias");
+  // long chunks with keys up to 128 wide: two value columns per lane (half the LDS reads per FMA, 2 DK / 4 state
+  // registers); one-token rows and short portions: one column, twice the workgroups
+  const int cpl = (max_q_len > 16 && vdim > 64 && dim <= 128) ? 2 : 1;
+  const dim3 grid(seqs, H, (vdim + 64 * cpl - 1) / (64 * cpl));
   hipStream_t s = (hipStream_t)stream;
-#define DR_SCAN(DK)                                                                                              \
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK>), grid, dim3(256), 0, s, (float*)o, (const float*)u, ld, \
-                     (const float*)bd, (float*)state, (const int32_t*)cu, (const int32_t*)positions,             \
+#define DR_SCAN(DK, TY)                                                                                              \
+  if (cpl == 2 && DK <= 128)                                                                                         \
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<(DK <= 128 ? DK : 128), 2, TY>), grid, dim3(256), 0, s, (float*)o, (const float*)u, ld, \
+                     (const float*)bd, (const void*)ab, ldab, bcol, (const float*)a_log, (const float*)dt_bias,      \
+                     qscale, unit_eps, (float*)state, (const int32_t*)cu, (const int32_t*)positions,                 \
+                     (const int32_t*)slots, H, G, dim, vdim);                                                        \
+  else                                                                                                               \
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, TY>), grid, dim3(256), 0, s, (float*)o, (const float*)u, ld, \
+                     (const float*)bd, (const void*)ab, ldab, bcol, (const float*)a_log, (const float*)dt_bias,      \
+                     qscale, unit_eps, (float*)state, (const int32_t*)cu, (const int32_t*)positions,                 \
                      (const int32_t*)slots, H, G, dim, vdim)
-  if (dim <= 32) DR_SCAN(32);
-  else if (dim <= 64) DR_SCAN(64);
-  else if (dim <= 128) DR_SCAN(128);
-  else DR_SCAN(256);
+#define DR_SCAN_T(DK) do { if (f32) DR_SCAN(DK, float); else DR_SCAN(DK, bf16); } while (0)
+  if (dim <= 32) DR_SCAN_T(32);
+  else if (dim <= 64) DR_SCAN_T(64);
+  else if (dim <= 128) DR_SCAN_T(128);
+  else DR_SCAN_T(256);
+#undef DR_SCAN_T
 #undef DR_SCAN
   DLLM_HIP_CHECK(hipGetLastError());
 }

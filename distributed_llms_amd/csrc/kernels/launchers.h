@@ -137,8 +137,9 @@ void relu_sq(uintptr_t y, long n, int f32, uintptr_t stream);
 // gated delta rule (delta.hip): everything float32 but the gate, the norm weight and the normed output
 void dr_prep(uintptr_t u, long ld, uintptr_t ab, long ldab, int bcol, uintptr_t a_log, uintptr_t dt_bias, uintptr_t bd,
              int tokens, int H, int G, int dim, float qscale, float unit_eps, int f32, uintptr_t stream);
-void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t state, uintptr_t cu, uintptr_t positions,
-             uintptr_t slots, int seqs, int H, int G, int dim, int vdim, uintptr_t stream);
+void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long ldab, int bcol, uintptr_t a_log,
+             uintptr_t dt_bias, float qscale, float unit_eps, uintptr_t state, uintptr_t cu, uintptr_t positions,
+             uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, int f32, uintptr_t stream);
 void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
                  int vdim, float eps, float out_scale, int f32, uintptr_t stream);
 void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,

@@ -983,7 +983,14 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_kernel(
     void* __restrict__ v_cache_, const int32_t* __restrict__ slot_mapping, const int32_t* __restrict__ positions, int H,
     int G, int D, int Dv, int bs) {
   __shared__ float red[16];
+  extern __shared__ float csn[];                   // cos | sin of the token's nrot angles
   const int t = blockIdx.x, tid = threadIdx.x;
+  const float fpos = (float)positions[t];
+  for (int i = tid; i < nrot; i += 256) {
+    const float ang = fpos * freqs[i];
+    csn[i] = cosf(ang);
+    csn[nrot + i] = sinf(ang);
+  }
   const T* q = (const T*)qkv_ + (size_t)t * ld + col0;
   const T* k = q + (size_t)H * D;
   const T* v = k + (size_t)G * D;
@@ -996,7 +1003,6 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_kernel(
   sq = block_sum(sq, red);
   sk = block_sum(sk, red);
   const float iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
-  const float fpos = (float)positions[t];
   const int slot = slot_mapping[t], blk = slot / bs, off = slot - blk * bs;
   T* q_out = (T*)q_out_ + (size_t)t * nq;
   T* kc = (T*)k_cache_;
@@ -1013,12 +1019,84 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_kernel(
       const int i = d < nrot ? d : d - nrot;
       const int pe = d < nrot ? ee + nrot : ee - nrot;          // the pair's other dimension
       const float y = ldf(src + pe) * inv * ldf(w + pe);
-      const float ang = fpos * freqs[i];
-      const float cs = cosf(ang), sn = sinf(ang);
+      const float cs = csn[i], sn = csn[nrot + i];
       x = d < nrot ? x * cs - y * sn : x * cs + y * sn;
     }
     if (isq) stf(q_out + ee, x);
     else stf(kc + (((size_t)blk * G + hd) * bs + off) * D + d, x);
+  }
+  for (int e = tid; e < nv; e += 256) {
+    const int g = e / Dv, c = e - g * Dv;
+    vc[(((size_t)blk * G + g) * Dv + c) * bs + off] = v[e];
+  }
+}
+
+// The same with 8 consecutive dimensions per lane (16-byte loads and stores for bf16): head size, rotated
+// half, row stride and first column are multiples of 8, so a lane's 8 dimensions and their 8 partners are
+// one aligned piece each.
+template <typename T>
+__global__ void __launch_bounds__(256) sm_rownorm_rope_vec_kernel(
+    void* __restrict__ q_out_, const void* __restrict__ qkv_, long ld, int col0, const void* __restrict__ qw_,
+    const void* __restrict__ kw_, const float* __restrict__ freqs, int nrot, float eps, void* __restrict__ k_cache_,
+    void* __restrict__ v_cache_, const int32_t* __restrict__ slot_mapping, const int32_t* __restrict__ positions, int H,
+    int G, int D, int Dv, int bs) {
+  __shared__ float red[32];
+  extern __shared__ float csn[];                   // cos | sin of the token's nrot angles
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const float fpos = (float)positions[t];
+  for (int i = tid; i < nrot; i += 256) {
+    const float ang = fpos * freqs[i];
+    csn[i] = cosf(ang);
+    csn[nrot + i] = sinf(ang);
+  }
+  const T* q = (const T*)qkv_ + (size_t)t * ld + col0;
+  const int nq = H * D, nk = G * D, nv = G * Dv;
+  const T* v = q + nq + nk;
+  float sq = 0.f, sk = 0.f;
+  for (int e = tid * 8; e < nq + nk; e += 2048) {
+    float x[8];
+    ldv<8>(q + e, x);
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a += x[i] * x[i];
+    if (e < nq) sq += a; else sk += a;
+  }
+  sq = wave_sum(sq);
+  sk = wave_sum(sk);
+  if (lane == 0) red[wid] = sq, red[4 + wid] = sk;
+  __syncthreads();                                 // also: csn is complete
+  sq = red[0] + red[1] + red[2] + red[3];
+  sk = red[4] + red[5] + red[6] + red[7];
+  const float iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
+  const int slot = slot_mapping[t], blk = slot / bs, off = slot - blk * bs;
+  T* q_out = (T*)q_out_ + (size_t)t * nq;
+  T* kc = (T*)k_cache_;
+  T* vc = (T*)v_cache_;
+  for (int e = tid * 8; e < nq + nk; e += 2048) {
+    const bool isq = e < nq;
+    const int ee = isq ? e : e - nq;
+    const T* w = (isq ? (const T*)qw_ : (const T*)kw_) + ee;
+    const float inv = isq ? iq : ik;
+    const int hd = ee / D, d = ee - hd * D;
+    float x[8], g[8];
+    ldv<8>(q + e, x);
+    ldv<8>(w, g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] *= inv * g[i];
+    if (d < 2 * nrot) {
+      const bool first = d < nrot;
+      const int po = first ? nrot : -nrot, i0 = first ? d : d - nrot;
+      float y[8], gy[8];
+      ldv<8>(q + e + po, y);
+      ldv<8>(w + po, gy);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float yy = y[i] * inv * gy[i], cs = csn[i0 + i], sn = csn[nrot + i0 + i];
+        x[i] = first ? x[i] * cs - yy * sn : x[i] * cs + yy * sn;
+      }
+    }
+    if (isq) stv<8>(q_out + ee, x);
+    else stv<8>(kc + (((size_t)blk * G + hd) * bs + off) * D + d, x);
   }
   for (int e = tid; e < nv; e += 256) {
     const int g = e / Dv, c = e - g * Dv;
@@ -1034,7 +1112,15 @@ void sm_rownorm_rope(uintptr_t q_out, uintptr_t qkv, long ld, int col0, uintptr_
                       ld >= col0 + (long)H * D + (long)G * (D + Dv),
                   "rownorm_rope sizes");
   DLLM_HOST_CHECK(q_out && k_cache && v_cache && q_norm && k_norm && (nrot == 0 || freqs), "rownorm_rope arguments");
-  SM_DISPATCH(f32, sm_rownorm_rope_kernel, dim3(tokens), dim3(256), 0, stream, (void*)q_out, (const void*)qkv, ld, col0,
+  const int esz = f32 ? 4 : 2;
+  if (D % 8 == 0 && nrot % 8 == 0 && ld % 8 == 0 && col0 % 8 == 0 && qkv % (8 * esz) == 0 && q_norm % (8 * esz) == 0 &&
+      k_norm % (8 * esz) == 0 && q_out % (8 * esz) == 0 && k_cache % (8 * esz) == 0) {
+    SM_DISPATCH(f32, sm_rownorm_rope_vec_kernel, dim3(tokens), dim3(256), 2 * (size_t)nrot * sizeof(float), stream,
+                (void*)q_out, (const void*)qkv, ld, col0, (const void*)q_norm, (const void*)k_norm, (const float*)freqs, nrot,
+                eps, (void*)k_cache, (void*)v_cache, (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs);
+    return;
+  }
+  SM_DISPATCH(f32, sm_rownorm_rope_kernel, dim3(tokens), dim3(256), 2 * (size_t)nrot * sizeof(float), stream, (void*)q_out, (const void*)qkv, ld, col0,
               (const void*)q_norm, (const void*)k_norm, (const float*)freqs, nrot, eps, (void*)k_cache, (void*)v_cache,
               (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs);
 }

@@ -2,7 +2,8 @@
 size (``bench.py --hybrid``), random weights, one GPU: Tudilix (sliding-window attention + RG-LRU) beside
 a Llama-architecture model of the same width, layer count, feed-forward size, head size and K/V heads;
 Gikovik (latent attention + grouped-choice mixture of experts) beside a Mixtral-architecture model of the
-same width, layer count, heads, expert count and experts per token, with expert weights of equal size.  Every step goes through the engine's StageRunner (the trace
+same width, layer count, heads, expert count and experts per token, with expert weights of equal size;
+Zebutar (chunked attention beside a gated delta rule, SwiGLU experts) beside the same Mixtral model.  Every step goes through the engine's StageRunner (the trace
 replayer builds the batches): one step with ``batch`` prompts of ``prompt_len`` tokens (prefill),
 then ``gen_len`` steps of one token per sequence (decode)."""
 from __future__ import annotations
@@ -88,6 +89,25 @@ def mixtral_config(size: str, vocab: int = 32000) -> ModelConfig:
                        rope_theta=1000000.0, num_experts=e, experts_per_token=top)
 
 
+def zebutar_config(size: str, vocab: int = 32000) -> ModelConfig:
+    """Width, layers, heads, experts and experts per token of the Gikovik / Mixtral sizes; attention with the
+    Mixtral model's heads (a quarter as many K/V heads, 128-wide, half of every head rotated) inside chunks
+    of 2048 positions, beside a delta rule with as many 128 x 128 states as attention heads and half as many
+    q / k heads, 4-tap convolutions; layers 0 and 3 dense, the others mixtures of three-matrix experts of the
+    Mixtral model's size with a shared expert."""
+    w, nl, ff, h, _d, _dr, _dv, _r, _qr, e, top, ef = GIKOVIK_SIZES[size]
+    inter = -(-(2 * ef // 3) // 256) * 256
+    moe = {"kind": "moe", "expert": {"ff": inter}, "shared": {"ff": inter}, "router": {"experts": e, "top": top}}
+    mixer = {"left": {"heads": h, "kv_heads": max(1, h // 4), "dim": 128, "vdim": 128, "mask": {"size": 2048},
+                      "scale": 128 ** -0.5, "rot": {"base": 10000.0, "dims": 64}},
+             "right": {"heads": h, "kv_heads": max(1, h // 2), "dim": 128, "vdim": 128, "conv": 4},
+             "left_scale": 1.0, "right_scale": 1.0}
+    layers = [{"type": "parallel", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff} if i % 3 == 0 else moe}
+              for i in range(nl)]
+    return ModelConfig.from_hf_config({"architecture": "Zebutar", "vocab": vocab, "width": w, "norm": {"eps": 1e-6},
+                                       "layers": layers}, name=f"zebutar-{size}")
+
+
 def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps: int, tmp: str, graphs: bool):
     import os
     os.makedirs(tmp, exist_ok=True)
@@ -124,14 +144,15 @@ def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps:
     return batch * prompt_len / min(pre), batch * gen_len / min(dec)
 
 
-MAKERS = {"tudilix": hybrid_config, "llama": llama_config, "gikovik": gikovik_config, "mixtral": mixtral_config}
-PAIRS = {"tudilix": "llama", "gikovik": "mixtral"}
+MAKERS = {"tudilix": hybrid_config, "llama": llama_config, "gikovik": gikovik_config, "mixtral": mixtral_config,
+          "zebutar": zebutar_config}
+PAIRS = {"tudilix": "llama", "gikovik": "mixtral", "zebutar": "mixtral"}
 
 
 def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int = 32, reps: int = 2,
         tmp: str = "/tmp/dllm_hybrid_bench", models=("tudilix", "llama")) -> dict:
-    """``models``: which to run, of tudilix, llama, gikovik, mixtral; a layer-list model and its flat
-    counterpart (tudilix / llama, gikovik / mixtral) also get the ratio of their throughputs."""
+    """``models``: which to run, of tudilix, llama, gikovik, zebutar, mixtral; a layer-list model and its flat
+    counterpart (tudilix / llama, gikovik / mixtral, zebutar / mixtral) also get the ratio of their throughputs."""
     out = {"size": size, "batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
            "data": "synthetic (random-init weights, random token ids)"}
     for key in models:

@@ -12,6 +12,7 @@ kv_heads)`` serves value head h.  The pieces, each an op of its own:
   :func:`unit_qk_gates`    q and k to unit length (q also times dim^-1/2), beta = sigmoid(b),
                            g = exp(-exp(A_log) softplus(a + dt_bias))
   :func:`delta_scan`       the recurrence over a varlen batch, state slots read and written
+  :func:`delta_scan_raw`   both of the above in one pass (what the mixer runs)
   :func:`gated_head_norm`  o / rms(o) * w * silu(gate) per head
 
 Same dispatch as the other ops: CUDA tensors go to the in-tree HIP kernels (csrc/kernels/delta.hip) and
@@ -28,6 +29,7 @@ from .seqmix import SeqBatch, _ck, _f32flag, _k, _stream
 
 UNIT_EPS = 1e-6          # inside the root of the unit norms: x / sqrt(sum(x^2) + UNIT_EPS)
 MAX_KEY_DIM = 256        # the scan kernel keeps a state column in registers
+FUSED_PREP_MAX_TOKENS = 16   # up to this many tokens per sequence the scan norms q / k and makes the gates itself
 
 
 @dataclass
@@ -108,8 +110,35 @@ def delta_scan(u: torch.Tensor, bd: torch.Tensor, state: torch.Tensor, sb: SeqBa
     _ck(bd, "bd", torch.float32)
     _ck(state, "state", torch.float32)
     o = torch.empty(t, hh, dv, dtype=torch.float32, device=u.device)
-    _k().dr_scan(o.data_ptr(), u.data_ptr(), u.shape[1], bd.data_ptr(), state.data_ptr(), sb.cu.data_ptr(),
-                 sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, hh, g, d, dv, _stream())
+    _k().dr_scan(o.data_ptr(), u.data_ptr(), u.shape[1], bd.data_ptr(), 0, 0, 0, 0, 0, 1.0, 0.0, state.data_ptr(),
+                 sb.cu.data_ptr(), sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, sb.max_q_len, hh, g, d,
+                 dv, 0, _stream())
+    return o
+
+
+def delta_scan_raw(u: torch.Tensor, ab: torch.Tensor, bcol: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                   state: torch.Tensor, sb: SeqBatch, spec: DeltaSpec, unit_eps: float = UNIT_EPS) -> torch.Tensor:
+    """:func:`unit_qk_gates` and :func:`delta_scan` in one pass: ``u`` holds the RAW q | k | v (after
+    convolution and activation; left unchanged), ``ab`` [T, *] the logits b | a from column ``bcol``; the GPU
+    kernel norms q and k and makes the gates on the tokens it stages for the recurrence."""
+    if not u.is_cuda:
+        u = u.clone()
+        return delta_scan(u, unit_qk_gates(u, ab, bcol, a_log, dt_bias, spec, unit_eps), state, sb, spec)
+    t = u.shape[0]
+    hh, g, d, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    if state.shape[1:] != (hh, d, dv) or state.dtype != torch.float32 or u.shape[1] != spec.conv_width or (
+            ab.shape[1] < bcol + 2 * hh) or d > MAX_KEY_DIM:
+        raise ValueError("delta_scan_raw: shape / dtype mismatch")
+    _ck(u, "u", torch.float32)
+    _ck(ab, "ab")
+    _ck(a_log, "a_log", torch.float32)
+    _ck(dt_bias, "dt_bias", torch.float32)
+    _ck(state, "state", torch.float32)
+    o = torch.empty(t, hh, dv, dtype=torch.float32, device=u.device)
+    _k().dr_scan(o.data_ptr(), u.data_ptr(), u.shape[1], 0, ab.data_ptr(), ab.shape[1], int(bcol), a_log.data_ptr(),
+                 dt_bias.data_ptr(), d ** -0.5, float(unit_eps), state.data_ptr(), sb.cu.data_ptr(),
+                 sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, sb.max_q_len, hh, g, d, dv,
+                 _f32flag(ab), _stream())
     return o
 
 
@@ -142,6 +171,11 @@ def gated_delta_mixer(proj: torch.Tensor, col0: int, w: dict, spec: DeltaSpec, c
     from . import seqmix as sm
     c = spec.conv_width
     u = sm.causal_conv(proj[:, col0:col0 + c], w["conv_w"], None, conv_state, sb, out_dtype=torch.float32, act="silu")
-    bd = unit_qk_gates(u, proj, col0 + c + spec.heads * spec.vdim, w["a_log"], w["dt_bias"], spec)
-    o = delta_scan(u, bd, state, sb, spec)
+    bcol = col0 + c + spec.heads * spec.vdim
+    if u.is_cuda and sb.max_q_len > FUSED_PREP_MAX_TOKENS:
+        # long chunks: the norms and gates as a pass of their own (in the scan they would be redone by every
+        # workgroup of a head, on the LDS path that bounds it)
+        o = delta_scan(u, unit_qk_gates(u, proj, bcol, w["a_log"], w["dt_bias"], spec), state, sb, spec)
+    else:
+        o = delta_scan_raw(u, proj, bcol, w["a_log"], w["dt_bias"], state, sb, spec)
     return gated_head_norm(o, proj, col0 + c, w["norm"], eps, out_scale)
