@@ -60,15 +60,16 @@ void dr_prep(uintptr_t u, long ld, uintptr_t ab, long ldab, int bcol, uintptr_t 
 // The recurrence.  Lane (part = lane / 16, jj = lane % 16) of wave w owns rows [part DK/4, (part + 1) DK/4) of
 // value column j = 64 z + 16 w + jj of the state of head h: S^T k and S^T q are DK/4 FMAs and a sum over the
 // four parts.  k and q (zero-padded to DK) and the gates of kDrTB tokens are staged in LDS for the
-// workgroup's four waves; the next block's global loads are issued before the current block's steps and
+// workgroup's NT / 64 waves (fewer waves and value columns per workgroup when few sequences and heads would
+// leave CUs idle: the chain of a token's steps, not the arithmetic, bounds a lone wave); the next block's global loads are issued before the current block's steps and
 // land in LDS after them.  With `ab_` the kernel takes the RAW q and k (after convolution and activation)
 // and the gate logits and does dr_prep_kernel's work on the staged block itself (unit norms, beta, g), so
 // the mixer needs no pass of its own for them.  A chunk that starts at position 0 starts from a zero
 // state; the state goes back to its slot after the chunk's last token.
 constexpr int kDrTB = 8;
 
-template <int DK, int CPL, typename T>
-__global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, const float* __restrict__ u, long ld,
+template <int DK, int CPL, int NT, typename T>
+__global__ void __launch_bounds__(NT) dr_scan_kernel(float* __restrict__ o, const float* __restrict__ u, long ld,
                                                       const float* __restrict__ bd, const void* __restrict__ ab_,
                                                       long ldab, int bcol, const float* __restrict__ a_log,
                                                       const float* __restrict__ dt_bias, float qscale, float unit_eps,
@@ -77,7 +78,8 @@ __global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, con
                                                       const int32_t* __restrict__ slots, int H, int G, int dim,
                                                       int vdim) {
   constexpr int R = DK / 4;
-  constexpr int NST = kDrTB * 2 * DK / 256;                   // staged k / q elements per thread and block
+  constexpr int NST = kDrTB * 2 * DK / NT;                    // staged k / q elements per thread and block
+  constexpr int NW = NT / 64;                                 // waves: 16 NW CPL value columns per workgroup
   __shared__ __attribute__((aligned(16))) float kq[kDrTB][2][DK];
   __shared__ float gates[kDrTB][2];
   const int b = blockIdx.x, h = blockIdx.y;
@@ -90,7 +92,7 @@ __global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, con
   bool jok[CPL];
 #pragma unroll
   for (int c = 0; c < CPL; ++c) {
-    j[c] = (blockIdx.z * CPL + c) * 64 + wave * 16 + jj;
+    j[c] = (blockIdx.z * CPL + c) * (16 * NW) + wave * 16 + jj;
     jok[c] = j[c] < vdim;
   }
   const int g = h / (H / G);
@@ -112,7 +114,7 @@ __global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, con
     const int nt = min(kDrTB, n - t0);
 #pragma unroll
     for (int r = 0; r < NST; ++r) {
-      const int idx = tid + 256 * r;
+      const int idx = tid + NT * r;
       const int tt = idx / (2 * DK), rem = idx - tt * 2 * DK, which = rem / DK, i = rem - which * DK;
       st[r] = (tt < nt && i < dim) ? u[(size_t)(lo + t0 + tt) * ld + (which ? qcol : kcol) + i] : 0.f;
     }
@@ -133,7 +135,7 @@ __global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, con
     __syncthreads();                                          // the previous block's reads are done
 #pragma unroll
     for (int r = 0; r < NST; ++r) {
-      const int idx = tid + 256 * r;
+      const int idx = tid + NT * r;
       (&kq[0][0][0])[idx] = st[r];
     }
     if (tid < nt * 2) {
@@ -148,7 +150,7 @@ __global__ void __launch_bounds__(256) dr_scan_kernel(float* __restrict__ o, con
       for (int tt = 0; tt < kDrTB; ++tt) vv[c][tt] = vn[c][tt];
     if (ab) {                                                 // unit norms of the staged k and q vectors
       __syncthreads();
-      for (int vec = wave; vec < nt * 2; vec += 4) {
+      for (int vec = wave; vec < nt * 2; vec += NW) {
         float* x = &kq[0][0][0] + vec * DK;
         float ss = 0.f;
         for (int i = lane; i < DK; i += 64) ss += x[i] * x[i];
@@ -220,21 +222,30 @@ void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long
   DLLM_HOST_CHECK((bd != 0) != (ab != 0) && (!ab || (a_log && dt_bias && ldab >= bcol + 2L * H && bcol >= 0)),
                   "delta rule gates: beta | g, or the raw logits with A_log and dt_bias");
   // long chunks with keys up to 128 wide: two value columns per lane (half the LDS reads per FMA, 2 DK / 4 state
-  // registers); one-token rows and short portions: one column, twice the workgroups
-  const int cpl = (max_q_len > 16 && vdim > 64 && dim <= 128) ? 2 : 1;
-  const dim3 grid(seqs, H, (vdim + 64 * cpl - 1) / (64 * cpl));
+  // registers); one-token rows and short portions: one column, twice the workgroups; and while the grid
+  // leaves CUs idle, fewer waves (value columns) per workgroup
+  int cpl = (max_q_len > 16 && vdim > 64 && dim <= 128) ? 2 : 1;
+  if ((long)seqs * H * ((vdim + 127) / 128) < 256) cpl = 1;
+  int nt = 256;
+  while (nt > 64 && vdim > nt / 8 && (long)seqs * H * ((vdim + nt / 4 - 1) / (nt / 4)) < 512) nt /= 2;
+  const int cols = cpl * nt / 4;
+  const dim3 grid(seqs, H, (vdim + cols - 1) / cols);
   hipStream_t s = (hipStream_t)stream;
-#define DR_SCAN(DK, TY)                                                                                              \
-  if (cpl == 2 && DK <= 128)                                                                                         \
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<(DK <= 128 ? DK : 128), 2, TY>), grid, dim3(256), 0, s, (float*)o, (const float*)u, ld, \
-                     (const float*)bd, (const void*)ab, ldab, bcol, (const float*)a_log, (const float*)dt_bias,      \
-                     qscale, unit_eps, (float*)state, (const int32_t*)cu, (const int32_t*)positions,                 \
-                     (const int32_t*)slots, H, G, dim, vdim);                                                        \
-  else                                                                                                               \
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, TY>), grid, dim3(256), 0, s, (float*)o, (const float*)u, ld, \
-                     (const float*)bd, (const void*)ab, ldab, bcol, (const float*)a_log, (const float*)dt_bias,      \
-                     qscale, unit_eps, (float*)state, (const int32_t*)cu, (const int32_t*)positions,                 \
-                     (const int32_t*)slots, H, G, dim, vdim)
+#define DR_ARGS                                                                                                   \
+  (float*)o, (const float*)u, ld, (const float*)bd, (const void*)ab, ldab, bcol, (const float*)a_log,             \
+      (const float*)dt_bias, qscale, unit_eps, (float*)state, (const int32_t*)cu, (const int32_t*)positions,      \
+      (const int32_t*)slots, H, G, dim, vdim
+#define DR_SCAN(DK, TY)                                                                                           \
+  do {                                                                                                            \
+    if (cpl == 2)                                                                                                 \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<(DK <= 128 ? DK : 128), 2, 256, TY>), grid, dim3(256), 0, s, DR_ARGS); \
+    else if (nt == 256)                                                                                           \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 256, TY>), grid, dim3(256), 0, s, DR_ARGS);       \
+    else if (nt == 128)                                                                                           \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 128, TY>), grid, dim3(128), 0, s, DR_ARGS);       \
+    else                                                                                                          \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 64, TY>), grid, dim3(64), 0, s, DR_ARGS);         \
+  } while (0)
 #define DR_SCAN_T(DK) do { if (f32) DR_SCAN(DK, float); else DR_SCAN(DK, bf16); } while (0)
   if (dim <= 32) DR_SCAN_T(32);
   else if (dim <= 64) DR_SCAN_T(64);
@@ -242,6 +253,7 @@ void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long
   else DR_SCAN_T(256);
 #undef DR_SCAN_T
 #undef DR_SCAN
+#undef DR_ARGS
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
