@@ -65,6 +65,8 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("sm_embed_norm", &dllm::sm_embed_norm);
   m.def("sm_rownorm_rope", &dllm::sm_rownorm_rope);
   m.def("dr_prep", &dllm::dr_prep);
+  m.def("dr_conv_prep", &dllm::dr_conv_prep);
+  m.def("sm_conv_tail", &dllm::sm_conv_tail);
   m.def("dr_scan", &dllm::dr_scan);
   m.def("dr_out_norm", &dllm::dr_out_norm);
   m.def("moe_combine_gated", &dllm::moe_combine_gated);

@@ -7,10 +7,11 @@
 //
 //   dr_prep_kernel      per token: q and k of every K/V head to unit length (q also times `qscale`), beta =
 //                       sigmoid(b), g = exp(-exp(A_log) softplus(a + dt_bias))
+//   dr_conv_prep_kernel the same behind the short convolutions + silu of q | k | v, one launch from the fused
+//                       projection (what the mixer runs)
 //   dr_scan_kernel      the recurrence over a varlen batch: a workgroup per (sequence, head, 64 value
 //                       columns); a column's state is thread-local (split over 4 lanes along dim), so a
-//                       step costs no exchange besides two 4-lane sums; optionally with dr_prep_kernel's
-//                       work done on the staged tokens (the product path)
+//                       step costs no exchange besides two 4-lane sums
 //   dr_out_norm_kernel  per (token, head): o / rms(o) * w * silu(gate)
 #include <math.h>
 
@@ -57,23 +58,90 @@ void dr_prep(uintptr_t u, long ld, uintptr_t ab, long ldab, int bcol, uintptr_t 
               (const float*)a_log, (const float*)dt_bias, (float*)bd, H, G, dim, qscale, unit_eps);
 }
 
+// The mixer's input stage in one launch, a workgroup per token: the causal convolutions of q | k | v (columns
+// col0 .. of the projection `x`, weights [taps, C] tap-major, tail in `state`, see sm_causal_conv_kernel) with
+// silu, then dr_prep_kernel's work on the result -- unit q and k (held in LDS between the two phases: 2 G dim
+// floats), beta and g -- into u [T, C] float32 and bd [T, 2 H].  The tail update stays a launch of its own
+// (sm_conv_tail): it must see every token's rows unchanged.
+template <typename T, int V>
+__global__ void __launch_bounds__(256) dr_conv_prep_kernel(
+    float* __restrict__ u, float* __restrict__ bd, const void* __restrict__ x_, long ld, int col0, int bcol,
+    const void* __restrict__ w_, const void* __restrict__ state_, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, const int32_t* __restrict__ cu, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ slots, int H, int G, int dim, int vdim, int taps,
+    float qscale, float unit_eps) {
+  extern __shared__ float qk[];                    // [2 G dim]
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = tok_seq[t];
+  const int tl = t - cu[b], pos = positions[t];
+  const int nqk = 2 * G * dim, C = nqk + H * vdim;
+  const T* x = (const T*)x_ + col0;
+  const T* w = (const T*)w_;
+  const T* st = (const T*)state_ + (size_t)slots[b] * (taps - 1) * C;
+  float* row = u + (size_t)t * C;
+  for (int c = tid * V; c < C; c += 256 * V) {
+    float acc[V], xv[V], wv[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      if (!conv_input_v<T, V>(x, ld, st, t, tl, pos, taps - 1 - j, taps, c, C, xv)) continue;
+      ldv<V>(w + (size_t)j * C + c, wv);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += wv[e] * xv[e];
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
+    if (c < nqk) stv<V>(qk + c, acc);              // V divides dim: a piece lies in one part
+    else stv<V>(row + c, acc);
+  }
+  __syncthreads();
+  for (int unit = wave; unit < 2 * G; unit += 4) {          // units 0 .. G - 1: q heads, G .. 2 G - 1: k heads
+    const float* xq = qk + (size_t)unit * dim;
+    float ss = 0.f;
+    for (int i = lane; i < dim; i += 64) ss += xq[i] * xq[i];
+    ss = wave_sum(ss);
+    const float m = (unit < G ? qscale : 1.0f) / sqrtf(ss + unit_eps);
+    for (int i = lane; i < dim; i += 64) row[(size_t)unit * dim + i] = xq[i] * m;
+  }
+  const T* ab = (const T*)x_ + (size_t)t * ld + bcol;
+  for (int h = tid; h < H; h += 256) {
+    bd[(size_t)t * 2 * H + h] = dr_sigmoid(ldf(ab + h));
+    bd[(size_t)t * 2 * H + H + h] = expf(-expf(a_log[h]) * dr_softplus(ldf(ab + H + h) + dt_bias[h]));
+  }
+}
+
+void dr_conv_prep(uintptr_t u, uintptr_t bd, uintptr_t x, long ld, int col0, int bcol, uintptr_t w, uintptr_t state,
+                  uintptr_t a_log, uintptr_t dt_bias, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
+                  int tokens, int H, int G, int dim, int vdim, int taps, float qscale, float unit_eps, int f32,
+                  uintptr_t stream) {
+  if (tokens <= 0) return;
+  const long C = 2L * G * dim + (long)H * vdim;
+  DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && dim > 0 && vdim > 0 && taps >= 1 && col0 >= 0 && bcol >= 0 &&
+                      ld >= col0 + C && ld >= bcol + 2L * H,
+                  "delta rule input stage sizes");
+  const size_t lds = sizeof(float) * 2 * (size_t)G * dim;
+  DLLM_HOST_CHECK(lds <= 48 * 1024, "delta rule input stage: q | k too wide for LDS");
+  const int esz = f32 ? 4 : 2;
+  const int vec = dim % 8 == 0 && vdim % 8 == 0 && ld % 8 == 0 && col0 % 8 == 0 && (x % (8 * esz)) == 0 &&
+                  (w % (8 * esz)) == 0 && (state % (8 * esz)) == 0;
+  SM_DISPATCH_V(f32, vec, dr_conv_prep_kernel, dim3(tokens), dim3(256), lds, stream, (float*)u, (float*)bd,
+                (const void*)x, ld, col0, bcol, (const void*)w, (const void*)state, (const float*)a_log,
+                (const float*)dt_bias, (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq,
+                (const int32_t*)slots, H, G, dim, vdim, taps, qscale, unit_eps);
+}
+
 // The recurrence.  Lane (part = lane / 16, jj = lane % 16) of wave w owns rows [part DK/4, (part + 1) DK/4) of
 // value column j = 64 z + 16 w + jj of the state of head h: S^T k and S^T q are DK/4 FMAs and a sum over the
 // four parts.  k and q (zero-padded to DK) and the gates of kDrTB tokens are staged in LDS for the
 // workgroup's NT / 64 waves (fewer waves and value columns per workgroup when few sequences and heads would
 // leave CUs idle: the chain of a token's steps, not the arithmetic, bounds a lone wave); the next block's global loads are issued before the current block's steps and
-// land in LDS after them.  With `ab_` the kernel takes the RAW q and k (after convolution and activation)
-// and the gate logits and does dr_prep_kernel's work on the staged block itself (unit norms, beta, g), so
-// the mixer needs no pass of its own for them.  A chunk that starts at position 0 starts from a zero
-// state; the state goes back to its slot after the chunk's last token.
+// land in LDS after them.  A chunk that starts at position 0 starts from a zero state; the state goes back
+// to its slot after the chunk's last token.
 constexpr int kDrTB = 8;
 
-template <int DK, int CPL, int NT, typename T>
+template <int DK, int CPL, int NT>
 __global__ void __launch_bounds__(NT) dr_scan_kernel(float* __restrict__ o, const float* __restrict__ u, long ld,
-                                                      const float* __restrict__ bd, const void* __restrict__ ab_,
-                                                      long ldab, int bcol, const float* __restrict__ a_log,
-                                                      const float* __restrict__ dt_bias, float qscale, float unit_eps,
-                                                      float* __restrict__ state, const int32_t* __restrict__ cu,
+                                                      const float* __restrict__ bd, float* __restrict__ state, const int32_t* __restrict__ cu,
                                                       const int32_t* __restrict__ positions,
                                                       const int32_t* __restrict__ slots, int H, int G, int dim,
                                                       int vdim) {
@@ -97,8 +165,6 @@ __global__ void __launch_bounds__(NT) dr_scan_kernel(float* __restrict__ o, cons
   }
   const int g = h / (H / G);
   const size_t kcol = (size_t)G * dim + (size_t)g * dim, qcol = (size_t)g * dim, vcol = 2 * (size_t)G * dim + (size_t)h * vdim;
-  const T* ab = (const T*)ab_;
-  const float ea = ab ? expf(a_log[h]) : 0.f, dtb = ab ? dt_bias[h] : 0.f;
   float* S = state + ((size_t)slots[b] * H + h) * dim * vdim;
   const bool fresh = positions[lo] == 0;
   float s[CPL][R];
@@ -125,8 +191,7 @@ __global__ void __launch_bounds__(NT) dr_scan_kernel(float* __restrict__ o, cons
         vn[c][tt] = (tt < nt && jok[c]) ? u[(size_t)(lo + t0 + tt) * ld + vcol + j[c]] : 0.f;
     if (tid < nt * 2) {
       const int tt = tid >> 1, w = tid & 1;
-      gn = ab ? ldf(ab + (size_t)(lo + t0 + tt) * ldab + bcol + w * H + h)
-              : bd[(size_t)(lo + t0 + tt) * 2 * H + w * H + h];
+      gn = bd[(size_t)(lo + t0 + tt) * 2 * H + w * H + h];
     }
   };
   fetch(0);
@@ -138,27 +203,12 @@ __global__ void __launch_bounds__(NT) dr_scan_kernel(float* __restrict__ o, cons
       const int idx = tid + NT * r;
       (&kq[0][0][0])[idx] = st[r];
     }
-    if (tid < nt * 2) {
-      float gv = gn;
-      if (ab) gv = (tid & 1) ? expf(-ea * dr_softplus(gn + dtb)) : dr_sigmoid(gn);
-      gates[tid >> 1][tid & 1] = gv;
-    }
+    if (tid < nt * 2) gates[tid >> 1][tid & 1] = gn;
     float vv[CPL][kDrTB];
 #pragma unroll
     for (int c = 0; c < CPL; ++c)
 #pragma unroll
       for (int tt = 0; tt < kDrTB; ++tt) vv[c][tt] = vn[c][tt];
-    if (ab) {                                                 // unit norms of the staged k and q vectors
-      __syncthreads();
-      for (int vec = wave; vec < nt * 2; vec += NW) {
-        float* x = &kq[0][0][0] + vec * DK;
-        float ss = 0.f;
-        for (int i = lane; i < DK; i += 64) ss += x[i] * x[i];
-        ss = wave_sum(ss);
-        const float m = ((vec & 1) ? qscale : 1.0f) / sqrtf(ss + unit_eps);
-        for (int i = lane; i < DK; i += 64) x[i] *= m;
-      }
-    }
     __syncthreads();
     if (t0 + kDrTB < n) fetch(t0 + kDrTB);
 #pragma unroll
@@ -210,17 +260,13 @@ __global__ void __launch_bounds__(NT) dr_scan_kernel(float* __restrict__ o, cons
     }
 }
 
-// `bd` [T, 2 H] (beta | g) with unit q and k in `u`, or -- bd null -- `ab` [T, ldab] in the activation type (f32:
-// float) holding the raw logits b | a from column `bcol`, with raw q and k in `u`.
-void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long ldab, int bcol, uintptr_t a_log,
-             uintptr_t dt_bias, float qscale, float unit_eps, uintptr_t state, uintptr_t cu, uintptr_t positions,
-             uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, int f32, uintptr_t stream) {
+// u [T, ld] float32: unit q | unit k | v; bd [T, 2 H]: beta | g.
+void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t state, uintptr_t cu, uintptr_t positions,
+             uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, uintptr_t stream) {
   if (seqs <= 0) return;
   DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && dim > 0 && dim <= 256 && vdim > 0 && H <= 65535 &&
                       ld >= 2L * G * dim + (long)H * vdim,
                   "delta rule sizes (key size up to 256)");
-  DLLM_HOST_CHECK((bd != 0) != (ab != 0) && (!ab || (a_log && dt_bias && ldab >= bcol + 2L * H && bcol >= 0)),
-                  "delta rule gates: beta | g, or the raw logits with A_log and dt_bias");
   // long chunks with keys up to 128 wide: two value columns per lane (half the LDS reads per FMA, 2 DK / 4 state
   // registers); one-token rows and short portions: one column, twice the workgroups; and while the grid
   // leaves CUs idle, fewer waves (value columns) per workgroup
@@ -232,26 +278,23 @@ void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long
   const dim3 grid(seqs, H, (vdim + cols - 1) / cols);
   hipStream_t s = (hipStream_t)stream;
 #define DR_ARGS                                                                                                   \
-  (float*)o, (const float*)u, ld, (const float*)bd, (const void*)ab, ldab, bcol, (const float*)a_log,             \
-      (const float*)dt_bias, qscale, unit_eps, (float*)state, (const int32_t*)cu, (const int32_t*)positions,      \
+  (float*)o, (const float*)u, ld, (const float*)bd, (float*)state, (const int32_t*)cu, (const int32_t*)positions, \
       (const int32_t*)slots, H, G, dim, vdim
-#define DR_SCAN(DK, TY)                                                                                           \
+#define DR_SCAN(DK)                                                                                               \
   do {                                                                                                            \
     if (cpl == 2)                                                                                                 \
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<(DK <= 128 ? DK : 128), 2, 256, TY>), grid, dim3(256), 0, s, DR_ARGS); \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<(DK <= 128 ? DK : 128), 2, 256>), grid, dim3(256), 0, s, DR_ARGS); \
     else if (nt == 256)                                                                                           \
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 256, TY>), grid, dim3(256), 0, s, DR_ARGS);       \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 256>), grid, dim3(256), 0, s, DR_ARGS);           \
     else if (nt == 128)                                                                                           \
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 128, TY>), grid, dim3(128), 0, s, DR_ARGS);       \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 128>), grid, dim3(128), 0, s, DR_ARGS);           \
     else                                                                                                          \
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 64, TY>), grid, dim3(64), 0, s, DR_ARGS);         \
+      hipLaunchKernelGGL(HIP_KERNEL_NAME(dr_scan_kernel<DK, 1, 64>), grid, dim3(64), 0, s, DR_ARGS);             \
   } while (0)
-#define DR_SCAN_T(DK) do { if (f32) DR_SCAN(DK, float); else DR_SCAN(DK, bf16); } while (0)
-  if (dim <= 32) DR_SCAN_T(32);
-  else if (dim <= 64) DR_SCAN_T(64);
-  else if (dim <= 128) DR_SCAN_T(128);
-  else DR_SCAN_T(256);
-#undef DR_SCAN_T
+  if (dim <= 32) DR_SCAN(32);
+  else if (dim <= 64) DR_SCAN(64);
+  else if (dim <= 128) DR_SCAN(128);
+  else DR_SCAN(256);
 #undef DR_SCAN
 #undef DR_ARGS
   DLLM_HIP_CHECK(hipGetLastError());

@@ -81,6 +81,8 @@ void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post
 void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,
                     uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
                     int tokens, int seqs, int C, int taps, int f32, int out_f32, int act, uintptr_t stream);
+void sm_conv_tail(uintptr_t state, uintptr_t u, long stride, uintptr_t cu, uintptr_t positions, uintptr_t slots, int seqs,
+                  int C, int taps, int f32, uintptr_t stream);
 void sm_rglru_gates(uintptr_t a, uintptr_t g, uintptr_t u, uintptr_t ra_t, uintptr_t ra_b, uintptr_t ri_t,
                     uintptr_t ri_b, uintptr_t lam, int tokens, int nb, int bw, float scale, int f32,
                     uintptr_t stream);
@@ -137,9 +139,12 @@ void relu_sq(uintptr_t y, long n, int f32, uintptr_t stream);
 // gated delta rule (delta.hip): everything float32 but the gate, the norm weight and the normed output
 void dr_prep(uintptr_t u, long ld, uintptr_t ab, long ldab, int bcol, uintptr_t a_log, uintptr_t dt_bias, uintptr_t bd,
              int tokens, int H, int G, int dim, float qscale, float unit_eps, int f32, uintptr_t stream);
-void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t ab, long ldab, int bcol, uintptr_t a_log,
-             uintptr_t dt_bias, float qscale, float unit_eps, uintptr_t state, uintptr_t cu, uintptr_t positions,
-             uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, int f32, uintptr_t stream);
+void dr_conv_prep(uintptr_t u, uintptr_t bd, uintptr_t x, long ld, int col0, int bcol, uintptr_t w, uintptr_t state,
+                  uintptr_t a_log, uintptr_t dt_bias, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
+                  int tokens, int H, int G, int dim, int vdim, int taps, float qscale, float unit_eps, int f32,
+                  uintptr_t stream);
+void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t state, uintptr_t cu, uintptr_t positions,
+             uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, uintptr_t stream);
 void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
                  int vdim, float eps, float out_scale, int f32, uintptr_t stream);
 void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,

@@ -195,27 +195,7 @@ void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post
 }
 
 // --------------------------------------------------------------------------- causal convolution with state
-// Input d rows before token (t, channel c) of a chunk that starts at position `start` with the token
-// at local index tl: the batch row t - d while tl - d >= 0, else the state tail row
-// tl - d + (taps - 1) while the position start + tl - d >= 0, else zero (before the sequence).
-// Weights are stored [taps, C] (tap-major), so V consecutive channels of one tap are one load.
-template <typename T>
-__device__ __forceinline__ float conv_input(const T* __restrict__ u, long stride, const T* __restrict__ st, int t,
-                                            int tl, int pos, int d, int taps, int c, int C) {
-  if (d > pos) return 0.f;
-  if (d <= tl) return ldf(u + (size_t)(t - d) * stride + c);
-  return ldf(st + (size_t)(tl - d + taps - 1) * C + c);
-}
-
-template <typename T, int V>
-__device__ __forceinline__ bool conv_input_v(const T* __restrict__ u, long stride, const T* __restrict__ st, int t,
-                                             int tl, int pos, int d, int taps, int c, int C, float (&o)[V]) {
-  if (d > pos) return false;
-  if (d <= tl) ldv<V>(u + (size_t)(t - d) * stride + c, o);
-  else ldv<V>(st + (size_t)(tl - d + taps - 1) * C + c, o);
-  return true;
-}
-
+// (conv_input / conv_input_v, the reads of a token's earlier inputs, are in stream_common.h)
 template <typename T, typename OT, int V>
 __global__ void __launch_bounds__(256) sm_causal_conv_kernel(void* __restrict__ y_, const void* __restrict__ u_,
                                                              long stride, const void* __restrict__ w_,
@@ -289,6 +269,16 @@ static void launch_conv_state(uintptr_t state, uintptr_t u, long stride, uintptr
   SM_DISPATCH_V(f32, vec, sm_conv_state_kernel, dim3(seqs, std::min(8, (C + per - 1) / per)), dim3(256), 0, stream,
                 (void*)state, (const void*)u, stride, (const int32_t*)cu, (const int32_t*)positions,
                 (const int32_t*)slots, C, taps);
+}
+
+// The tail update alone (a caller that ran the convolution in a kernel of its own).
+void sm_conv_tail(uintptr_t state, uintptr_t u, long stride, uintptr_t cu, uintptr_t positions, uintptr_t slots, int seqs,
+                  int C, int taps, int f32, uintptr_t stream) {
+  if (seqs <= 0 || taps <= 1) return;
+  DLLM_HOST_CHECK(C > 0 && stride >= C, "conv sizes");
+  const int esz = f32 ? 4 : 2;
+  launch_conv_state(state, u, stride, cu, positions, slots, seqs, C, taps, f32,
+                    C % 8 == 0 && stride % 8 == 0 && (u % (8 * esz)) == 0, stream);
 }
 
 void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,

@@ -66,6 +66,27 @@ template <int V> __device__ __forceinline__ void stv(float* p, const float (&o)[
   }
 }
 
+// Input d rows before token (t, channel c) of a chunk that starts at position `start` with the token
+// at local index tl: the batch row t - d while tl - d >= 0, else the state tail row
+// tl - d + (taps - 1) while the position start + tl - d >= 0, else zero (before the sequence).
+// Weights are stored [taps, C] (tap-major), so V consecutive channels of one tap are one load.
+template <typename T>
+__device__ __forceinline__ float conv_input(const T* __restrict__ u, long stride, const T* __restrict__ st, int t,
+                                            int tl, int pos, int d, int taps, int c, int C) {
+  if (d > pos) return 0.f;
+  if (d <= tl) return ldf(u + (size_t)(t - d) * stride + c);
+  return ldf(st + (size_t)(tl - d + taps - 1) * C + c);
+}
+
+template <typename T, int V>
+__device__ __forceinline__ bool conv_input_v(const T* __restrict__ u, long stride, const T* __restrict__ st, int t,
+                                             int tl, int pos, int d, int taps, int c, int C, float (&o)[V]) {
+  if (d > pos) return false;
+  if (d <= tl) ldv<V>(u + (size_t)(t - d) * stride + c, o);
+  else ldv<V>(st + (size_t)(tl - d + taps - 1) * C + c, o);
+  return true;
+}
+
 #define SM_DISPATCH(f32, KERNEL, grid, block, lds, stream, ...)                                        \
   do {                                                                                                 \
     if (f32)                                                                                           \

@@ -12,7 +12,8 @@ kv_heads)`` serves value head h.  The pieces, each an op of its own:
   :func:`unit_qk_gates`    q and k to unit length (q also times dim^-1/2), beta = sigmoid(b),
                            g = exp(-exp(A_log) softplus(a + dt_bias))
   :func:`delta_scan`       the recurrence over a varlen batch, state slots read and written
-  :func:`delta_scan_raw`   both of the above in one pass (what the mixer runs)
+  :func:`conv_unit_gates`  the same behind the short convolutions + silu, from the fused projection (what the
+                           mixer runs: one launch)
   :func:`gated_head_norm`  o / rms(o) * w * silu(gate) per head
 
 Same dispatch as the other ops: CUDA tensors go to the in-tree HIP kernels (csrc/kernels/delta.hip) and
@@ -29,7 +30,6 @@ from .seqmix import SeqBatch, _ck, _f32flag, _k, _stream
 
 UNIT_EPS = 1e-6          # inside the root of the unit norms: x / sqrt(sum(x^2) + UNIT_EPS)
 MAX_KEY_DIM = 256        # the scan kernel keeps a state column in registers
-FUSED_PREP_MAX_TOKENS = 16   # up to this many tokens per sequence the scan norms q / k and makes the gates itself
 
 
 @dataclass
@@ -110,36 +110,42 @@ def delta_scan(u: torch.Tensor, bd: torch.Tensor, state: torch.Tensor, sb: SeqBa
     _ck(bd, "bd", torch.float32)
     _ck(state, "state", torch.float32)
     o = torch.empty(t, hh, dv, dtype=torch.float32, device=u.device)
-    _k().dr_scan(o.data_ptr(), u.data_ptr(), u.shape[1], bd.data_ptr(), 0, 0, 0, 0, 0, 1.0, 0.0, state.data_ptr(),
-                 sb.cu.data_ptr(), sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, sb.max_q_len, hh, g, d,
-                 dv, 0, _stream())
+    _k().dr_scan(o.data_ptr(), u.data_ptr(), u.shape[1], bd.data_ptr(), state.data_ptr(), sb.cu.data_ptr(),
+                 sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, sb.max_q_len, hh, g, d, dv, _stream())
     return o
 
 
-def delta_scan_raw(u: torch.Tensor, ab: torch.Tensor, bcol: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
-                   state: torch.Tensor, sb: SeqBatch, spec: DeltaSpec, unit_eps: float = UNIT_EPS) -> torch.Tensor:
-    """:func:`unit_qk_gates` and :func:`delta_scan` in one pass: ``u`` holds the RAW q | k | v (after
-    convolution and activation; left unchanged), ``ab`` [T, *] the logits b | a from column ``bcol``; the GPU
-    kernel norms q and k and makes the gates on the tokens it stages for the recurrence."""
-    if not u.is_cuda:
-        u = u.clone()
-        return delta_scan(u, unit_qk_gates(u, ab, bcol, a_log, dt_bias, spec, unit_eps), state, sb, spec)
-    t = u.shape[0]
-    hh, g, d, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
-    if state.shape[1:] != (hh, d, dv) or state.dtype != torch.float32 or u.shape[1] != spec.conv_width or (
-            ab.shape[1] < bcol + 2 * hh) or d > MAX_KEY_DIM:
-        raise ValueError("delta_scan_raw: shape / dtype mismatch")
-    _ck(u, "u", torch.float32)
-    _ck(ab, "ab")
+def conv_unit_gates(proj: torch.Tensor, col0: int, conv_w: torch.Tensor, conv_state: torch.Tensor, a_log: torch.Tensor,
+                    dt_bias: torch.Tensor, sb: SeqBatch, spec: DeltaSpec, unit_eps: float = UNIT_EPS):
+    """The mixer's input stage from its fused projection ``proj`` [T, *] = .. | q | k | v | gate | b | a from
+    column ``col0``: the short causal convolutions of q | k | v (``conv_w`` [taps, conv_width] tap-major, tail in
+    ``conv_state`` [slots, taps - 1, conv_width], brought up to date) with silu, then :func:`unit_qk_gates`.
+    One launch (+ the tail update) on the GPU.  Returns (u [T, conv_width] float32, bd [T, 2 heads] float32)."""
+    from . import seqmix as sm
+    t = proj.shape[0]
+    c = spec.conv_width
+    bcol = col0 + c + spec.heads * spec.vdim
+    taps = conv_w.shape[0]
+    if proj.shape[1] < bcol + 2 * spec.heads or conv_w.shape != (spec.taps, c) or conv_state.shape[1:] != (taps - 1, c):
+        raise ValueError("conv_unit_gates: shape mismatch")
+    if not proj.is_cuda:
+        u = sm.causal_conv(proj[:, col0:col0 + c], conv_w, None, conv_state, sb, out_dtype=torch.float32, act="silu")
+        return u, unit_qk_gates(u, proj, bcol, a_log, dt_bias, spec, unit_eps)
+    _ck(proj, "proj")
+    _ck(conv_w, "conv_w", proj.dtype)
+    _ck(conv_state, "conv_state", proj.dtype)
     _ck(a_log, "a_log", torch.float32)
     _ck(dt_bias, "dt_bias", torch.float32)
-    _ck(state, "state", torch.float32)
-    o = torch.empty(t, hh, dv, dtype=torch.float32, device=u.device)
-    _k().dr_scan(o.data_ptr(), u.data_ptr(), u.shape[1], 0, ab.data_ptr(), ab.shape[1], int(bcol), a_log.data_ptr(),
-                 dt_bias.data_ptr(), d ** -0.5, float(unit_eps), state.data_ptr(), sb.cu.data_ptr(),
-                 sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, sb.max_q_len, hh, g, d, dv,
-                 _f32flag(ab), _stream())
-    return o
+    u = torch.empty(t, c, dtype=torch.float32, device=proj.device)
+    bd = torch.empty(t, 2 * spec.heads, dtype=torch.float32, device=proj.device)
+    f = _f32flag(proj)
+    _k().dr_conv_prep(u.data_ptr(), bd.data_ptr(), proj.data_ptr(), proj.shape[1], int(col0), int(bcol), conv_w.data_ptr(),
+                      conv_state.data_ptr(), a_log.data_ptr(), dt_bias.data_ptr(), sb.cu.data_ptr(), sb.positions.data_ptr(),
+                      sb.tok_seq.data_ptr(), sb.state_slots.data_ptr(), t, spec.heads, spec.kv_heads, spec.dim, spec.vdim,
+                      taps, spec.dim ** -0.5, float(unit_eps), f, _stream())
+    _k().sm_conv_tail(conv_state.data_ptr(), proj.data_ptr() + col0 * proj.element_size(), proj.shape[1], sb.cu.data_ptr(),
+                      sb.positions.data_ptr(), sb.state_slots.data_ptr(), sb.num_seqs, c, taps, f, _stream())
+    return u, bd
 
 
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, gcol: int, w: torch.Tensor, eps: float,
@@ -168,14 +174,7 @@ def gated_delta_mixer(proj: torch.Tensor, col0: int, w: dict, spec: DeltaSpec, c
     fused projection q | k | v | gate | b | a.  ``w``: ``conv_w`` [taps, conv_width] (tap-major), ``a_log`` and
     ``dt_bias`` [heads] float32, ``norm`` [vdim].  ``conv_state`` [slots, taps - 1, conv_width] holds the
     last inputs of the convolutions, ``state`` the matrices.  Returns [T, heads vdim]."""
-    from . import seqmix as sm
     c = spec.conv_width
-    u = sm.causal_conv(proj[:, col0:col0 + c], w["conv_w"], None, conv_state, sb, out_dtype=torch.float32, act="silu")
-    bcol = col0 + c + spec.heads * spec.vdim
-    if u.is_cuda and sb.max_q_len > FUSED_PREP_MAX_TOKENS:
-        # long chunks: the norms and gates as a pass of their own (in the scan they would be redone by every
-        # workgroup of a head, on the LDS path that bounds it)
-        o = delta_scan(u, unit_qk_gates(u, proj, bcol, w["a_log"], w["dt_bias"], spec), state, sb, spec)
-    else:
-        o = delta_scan_raw(u, proj, bcol, w["a_log"], w["dt_bias"], state, sb, spec)
+    u, bd = conv_unit_gates(proj, col0, w["conv_w"], conv_state, w["a_log"], w["dt_bias"], sb, spec)
+    o = delta_scan(u, bd, state, sb, spec)
     return gated_head_norm(o, proj, col0 + c, w["norm"], eps, out_scale)

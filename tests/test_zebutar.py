@@ -197,7 +197,7 @@ def _atol(dtype, f32=2e-5, bf16=3e-2):
 # ------------------------------------------------------------------------------ mechanisms alone
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("shape", [(4, 2, 56, 48, 16, 24), (6, 3, 32, 32, 32, 64), (3, 1, 20, 20, 16, 10), (2, 2, 64, 128, 32, 33),
-                                   (2, 1, 12, 12, 32, 1)])
+                                   (2, 1, 12, 12, 32, 1), (2, 1, 160, 192, 32, 40), (20, 1, 40, 40, 32, 70)])
 def test_keys_at_the_edges_of_a_chunk(target, shape):
     """Attention inside chunks of C positions.  One key gets a score far above the rest: (a) the first key
     of the query's chunk, the query anywhere in the chunk up to its last position -- it owns the output;
@@ -685,3 +685,42 @@ def test_decode_graphs_replay_like_eager_steps(target, tmp_path):
     graphed = replay(eng, sched, p)
     for n in p:
         np.testing.assert_allclose(graphed[n], eager[n], rtol=1e-3, atol=1e-3)
+
+
+def test_trace_run_program_loads_a_model_folder(tmp_path):
+    """bin/trace_run on a folder with config.json + model.safetensors (bfloat16): the registry picks the
+    stage by the config, the checkpoint loader reads the tensors, steps with portions beside single tokens
+    answer with the wanted logits (CPU path, float32)."""
+    import os
+    import subprocess
+    import sys
+    from safetensors.torch import save_file
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = cfg_a()
+    sd = {k: torch.from_numpy(v).to(torch.bfloat16) for k, v in O.make_weights(cfg, seed=21).items()}
+    model = tmp_path / "model"
+    model.mkdir()
+    (model / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in sd.items()}, str(model / "model.safetensors"))
+    rng = np.random.default_rng(3)
+    toks = {"a": rng.integers(0, cfg["vocab"], 50).tolist(), "b": rng.integers(0, cfg["vocab"], 21).tolist()}
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks["a"][:30], "want": [0, 29]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks["a"][30:31], "want": [0]},
+                                {"id": "b", "tokens": toks["b"][:20], "want": [19]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": toks["b"][20:], "want": []}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": toks["a"][31:], "want": [18]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(model), "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    assert not (out / "2.f32").exists()                       # nothing wanted in step 2
+    f64 = {k: v.double().numpy() for k, v in sd.items()}
+    ref = {n: O.forward(cfg, f64, t) for n, t in toks.items()}
+    got = {i: np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]) for i in (0, 1, 3)}
+    assert row_errs(got[0], ref["a"][[0, 29]]).max() < 1e-4
+    assert row_errs(got[1], np.stack([ref["a"][30], ref["b"][19]])).max() < 1e-4
+    assert row_errs(got[3], ref["a"][[49]]).max() < 1e-4
