@@ -1,8 +1,9 @@
 // Kernels of layer-list models with per-sequence state (ops/seqmix.py): a float32 residual stream
 // with RMS norms before and after every sublayer, short causal convolutions whose tail lives in a
 // state slot, the real-gated linear recurrent unit (gates, then a chunked linear scan), the
-// attention input stage (convolution + per-head norm + interleaved rotation + paged append), a
-// clipped GLU and the logit soft cap.
+// attention input stages (convolution + per-head norm + interleaved rotation + paged append; whole-
+// projection norm + half-split rotation + paged append), embedding + norm, a clipped GLU and the logit
+// soft cap.
 //
 // Every kernel is a template over the activation type T (bf16 or float): the float32 build is the
 // exact path (true 32-bit everywhere), the bf16 build keeps in float32 what feeds a norm, a

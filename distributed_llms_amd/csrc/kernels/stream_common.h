@@ -1,6 +1,7 @@
-// Helpers shared by the kernels of layer-list models (seqmix.hip, latent.hip): loads and stores of V
-// consecutive elements of the activation type T (bf16 or float) as float registers, and the launch
-// macros that pick the float32 or bf16 build of a kernel template.
+// Helpers shared by the kernels of layer-list models (seqmix.hip, latent.hip, delta.hip): loads and stores
+// of V consecutive elements of the activation type T (bf16 or float) as float registers, the reads of a
+// causal convolution's earlier inputs (batch rows, then the state tail, then zeros), and the launch macros
+// that pick the float32 or bf16 build of a kernel template.
 #pragma once
 #include <math.h>
 

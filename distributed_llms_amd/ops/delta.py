@@ -30,6 +30,7 @@ from .seqmix import SeqBatch, _ck, _f32flag, _k, _stream
 
 UNIT_EPS = 1e-6          # inside the root of the unit norms: x / sqrt(sum(x^2) + UNIT_EPS)
 MAX_KEY_DIM = 256        # the scan kernel keeps a state column in registers
+PREP_LDS_BYTES = 48 * 1024   # the fused input stage holds a token's q | k (float32) in LDS
 
 
 @dataclass
@@ -128,7 +129,8 @@ def conv_unit_gates(proj: torch.Tensor, col0: int, conv_w: torch.Tensor, conv_st
     taps = conv_w.shape[0]
     if proj.shape[1] < bcol + 2 * spec.heads or conv_w.shape != (spec.taps, c) or conv_state.shape[1:] != (taps - 1, c):
         raise ValueError("conv_unit_gates: shape mismatch")
-    if not proj.is_cuda:
+    if not proj.is_cuda or 8 * spec.kv_heads * spec.dim > PREP_LDS_BYTES:
+        # (on the GPU: q | k of a token wider than the fused kernel's LDS buffer -- the two mechanisms apart)
         u = sm.causal_conv(proj[:, col0:col0 + c], conv_w, None, conv_state, sb, out_dtype=torch.float32, act="silu")
         return u, unit_qk_gates(u, proj, bcol, a_log, dt_bias, spec, unit_eps)
     _ck(proj, "proj")

@@ -1,7 +1,9 @@
 """Ops of layer-list models whose layers carry per-sequence state: a float32 residual stream with
-pre- and post-sublayer RMS norms, short causal convolutions with a state tail, the real-gated linear
-recurrent unit (RG-LRU), sliding-window attention over a paged K/V cache whose key and value widths
-differ, a clipped GLU and the logit soft cap.
+pre- and post-sublayer RMS norms (also for sublayers that read the stream unnormed, and for two mixer
+outputs summed with scales), short causal convolutions with a state tail, the real-gated linear
+recurrent unit (RG-LRU), sliding-window and chunked attention over a paged K/V cache whose key and value
+widths differ, two attention input stages (convolution + per-head norm + interleaved rotation; whole-
+projection norm + half-split rotation), a clipped GLU and the logit soft cap.
 
 Same dispatch as :mod:`distributed_llms_amd.ops`: a CUDA tensor goes to the in-tree HIP kernels
 (csrc/kernels/seqmix.hip, attention_window.hip) and raises if they are not built; CPU tensors run
