@@ -95,13 +95,34 @@ __global__ void __launch_bounds__(256) dr_conv_prep_kernel(
     else stv<V>(row + c, acc);
   }
   __syncthreads();
-  for (int unit = wave; unit < 2 * G; unit += 4) {          // units 0 .. G - 1: q heads, G .. 2 G - 1: k heads
-    const float* xq = qk + (size_t)unit * dim;
-    float ss = 0.f;
-    for (int i = lane; i < dim; i += 64) ss += xq[i] * xq[i];
-    ss = wave_sum(ss);
-    const float m = (unit < G ? qscale : 1.0f) / sqrtf(ss + unit_eps);
-    for (int i = lane; i < dim; i += 64) row[(size_t)unit * dim + i] = xq[i] * m;
+  const int lpu = dim >> 3;                                 // lanes per unit when a lane takes 8 dimensions
+  if (V == 8 && lpu <= 64 && (lpu & (lpu - 1)) == 0) {
+    // units 0 .. G - 1: q heads, G .. 2 G - 1: k heads; 256 / lpu units per pass, each on an aligned lane group
+    for (int p0 = 0; p0 < nqk; p0 += 2048) {
+      const int c = p0 + tid * 8;
+      const bool ok = c < nqk;
+      float xv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[e] = 0.f;
+      if (ok) ldv<8>(qk + c, xv);
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += xv[e] * xv[e];
+      for (int m = lpu >> 1; m > 0; m >>= 1) ss += __shfl_xor(ss, m, 64);
+      const float m = (c < G * dim ? qscale : 1.0f) / sqrtf(ss + unit_eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[e] *= m;
+      if (ok) stv<8>(row + c, xv);
+    }
+  } else {
+    for (int unit = wave; unit < 2 * G; unit += 4) {
+      const float* xq = qk + (size_t)unit * dim;
+      float ss = 0.f;
+      for (int i = lane; i < dim; i += 64) ss += xq[i] * xq[i];
+      ss = wave_sum(ss);
+      const float m = (unit < G ? qscale : 1.0f) / sqrtf(ss + unit_eps);
+      for (int i = lane; i < dim; i += 64) row[(size_t)unit * dim + i] = xq[i] * m;
+    }
   }
   const T* ab = (const T*)x_ + (size_t)t * ld + bcol;
   for (int h = tid; h < H; h += 256) {
@@ -322,11 +343,48 @@ __global__ void __launch_bounds__(64) dr_out_norm_kernel(void* __restrict__ y_, 
   }
 }
 
+// The same with 8 channels per lane, vdim / 8 (a power of two) lanes per (token, head) on an aligned lane group.
+template <typename T>
+__global__ void __launch_bounds__(256) dr_out_norm_vec_kernel(void* __restrict__ y_, long ldy, const float* __restrict__ o,
+                                                             const void* __restrict__ gate_, long ldg, int gcol,
+                                                             const void* __restrict__ w_, long heads_total, int H,
+                                                             int vdim, float eps, float out_scale) {
+  const int lph = vdim >> 3;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const long th = idx / lph;
+  const int c = (int)(idx - th * lph) * 8;
+  const bool ok = th < heads_total;
+  const long thc = ok ? th : heads_total - 1;
+  const long t = thc / H;
+  const int h = (int)(thc - t * H);
+  float xv[8], gv[8], wv[8];
+  ldv<8>(o + (size_t)thc * vdim + c, xv);
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ss += xv[e] * xv[e];
+  for (int m = lph >> 1; m > 0; m >>= 1) ss += __shfl_xor(ss, m, 64);
+  const float inv = out_scale / sqrtf(ss / (float)vdim + eps);
+  ldv<8>((const T*)gate_ + (size_t)t * ldg + gcol + (size_t)h * vdim + c, gv);
+  ldv<8>((const T*)w_ + c, wv);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) xv[e] = xv[e] * inv * wv[e] * (gv[e] * dr_sigmoid(gv[e]));
+  if (ok) stv<8>((T*)y_ + (size_t)t * ldy + (size_t)h * vdim + c, xv);
+}
+
 void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
                  int vdim, float eps, float out_scale, int f32, uintptr_t stream) {
   if (tokens <= 0) return;
   DLLM_HOST_CHECK(H > 0 && H <= 65535 && vdim > 0 && ldy >= (long)H * vdim && ldg >= gcol + (long)H * vdim && gcol >= 0,
                   "delta rule output norm sizes");
+  const int esz = f32 ? 4 : 2, lph = vdim >> 3;
+  if (vdim % 8 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 && ldy % 8 == 0 && ldg % 8 == 0 && gcol % 8 == 0 &&
+      y % (8 * esz) == 0 && gate % (8 * esz) == 0 && w % (8 * esz) == 0 && o % 32 == 0) {
+    const long heads_total = (long)tokens * H, lanes = heads_total * lph;
+    DLLM_HOST_CHECK((lanes + 255) / 256 < (1L << 31), "delta rule output norm grid");
+    SM_DISPATCH(f32, dr_out_norm_vec_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream, (void*)y, ldy,
+                (const float*)o, (const void*)gate, ldg, gcol, (const void*)w, heads_total, H, vdim, eps, out_scale);
+    return;
+  }
   SM_DISPATCH(f32, dr_out_norm_kernel, dim3(tokens, H), dim3(64), 0, stream, (void*)y, ldy, (const float*)o,
               (const void*)gate, ldg, gcol, (const void*)w, H, vdim, eps, out_scale);
 }
