@@ -22,7 +22,7 @@ from typing import Any, Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2"; layer-list models: "tudilix", "gikovik", "zebutar"
+    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2"; layer-list models: "tudilix", "gikovik", "zebutar", "fekizen"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -49,6 +49,7 @@ class ModelConfig:
     # their weights (every repetition gets separate caches); and the width of the per-layer token input
     loop: Optional[Dict[str, int]] = None
     token_side_dim: int = 0
+    embed_scale: float = 1.0       # arch "fekizen": token embeddings enter times this; ``max_position`` rows of learned positions
 
     # ------------------------------------------------------------------ sizes
     @property
@@ -58,7 +59,7 @@ class ModelConfig:
     @property
     def needs_state_slots(self) -> bool:
         """Sequences carry per-layer state besides paged K/V (recurrent state, convolution tails)."""
-        return self.layers is not None and self.arch in ("tudilix", "zebutar")
+        return self.layers is not None and self.arch in ("tudilix", "zebutar", "fekizen")
 
     @property
     def needs_seq_index(self) -> bool:
@@ -133,6 +134,13 @@ class ModelConfig:
             if self.token_side_dim:
                 d["token_side"] = {"dim": self.token_side_dim}
             return d
+        if self.arch == "fekizen":
+            d = {"architecture": "Fekizen", "layers": [dict(l) for l in self.layers], "norm": {"eps": self.norm_eps},
+                 "vocab": self.vocab_size, "width": self.hidden_size, "embedding": {"scale": self.embed_scale},
+                 "max_positions": self.max_position, "_dllm_name": self.name}
+            if self.loop:
+                d["loop"] = dict(self.loop)
+            return d
         if self.arch == "zebutar":
             return {"architecture": "Zebutar", "layers": [dict(l) for l in self.layers], "norm": {"eps": self.norm_eps},
                     "vocab": self.vocab_size, "width": self.hidden_size, "_dllm_name": self.name}
@@ -178,6 +186,8 @@ class ModelConfig:
             return _from_gikovik(cfg, name)
         if cfg.get("architecture") == "Zebutar":
             return _from_zebutar(cfg, name)
+        if cfg.get("architecture") == "Fekizen":
+            return _from_fekizen(cfg, name)
         mt = cfg.get("model_type", "llama")
         name = name or cfg.get("_dllm_name") or cfg.get("_name_or_path") or mt
         eos = cfg.get("eos_token_id", 2)
@@ -293,6 +303,37 @@ def _from_zebutar(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelConfi
         norm_eps=float(cfg["norm"]["eps"]), bos_token_id=-1, eos_token_id=-1, layers=layers)
 
 
+def _from_fekizen(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelConfig:
+    """A ``config.json`` with "architecture": "Fekizen": ``width``, ``vocab``, ``norm.eps``, ``embedding.scale``,
+    ``max_positions`` (rows of the learned position table), ``layers`` (per layer ``type`` "lightning" |
+    "parallel", ``mixer`` sizes, ``mlp`` None | moe) and optionally ``loop`` (start, stop, times)."""
+    layers = [dict(l) for l in cfg["layers"]]
+    if not layers:
+        raise ValueError("layer-list config without layers")
+    for l in layers:
+        if l["type"] not in ("lightning", "parallel"):
+            raise ValueError(f"unsupported layer type {l['type']!r} (lightning, parallel)")
+        if l.get("mlp") is not None and l["mlp"].get("kind") != "moe":
+            raise ValueError(f"unsupported mlp kind {l['mlp'].get('kind')!r} (moe)")
+    extra = set(cfg.get("norm", {})) - {"eps"}
+    if extra:
+        raise ValueError(f"unsupported norm options {sorted(extra)}")
+    loop = cfg.get("loop")
+    if loop:
+        loop = {k: int(loop[k]) for k in ("start", "stop", "times")}
+        if not (0 <= loop["start"] < loop["stop"] <= len(layers)) or loop["times"] < 1:
+            raise ValueError(f"loop {loop} does not fit {len(layers)} layers")
+    left = [l["mixer"]["left"] for l in layers if l["type"] == "parallel"]
+    ff = [l["mlp"]["expert"]["ff"] for l in layers if l.get("mlp")]
+    return ModelConfig(
+        name=name or cfg.get("_dllm_name") or "fekizen", arch="fekizen", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), intermediate_size=int(max(ff or [0])), num_layers=len(layers),
+        num_heads=max([m["heads"] for m in left] or [1]), num_kv_heads=max([m["kv_heads"] for m in left] or [1]),
+        head_dim=max([max(m["dim"], m["vdim"]) for m in left] or [1]), max_position=int(cfg["max_positions"]),
+        norm_eps=float(cfg["norm"]["eps"]), bos_token_id=-1, eos_token_id=-1, layers=layers, loop=loop or None,
+        embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)))
+
+
 _LLAMA3_ROPE = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                 "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
 
@@ -388,6 +429,25 @@ PRESETS: Dict[str, ModelConfig] = {
                 "left_scale": 1.0, "right_scale": 1.0},
              "mlp": None},
         ]}, name="tiny-zebutar"),
+    "tiny-fekizen": _from_fekizen({
+        "architecture": "Fekizen", "vocab": 288, "width": 96, "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+        "max_positions": 1024, "loop": {"start": 1, "stop": 3, "times": 2},
+        "layers": [
+            {"type": "lightning", "mixer": {"heads": 3, "dim": 16, "vdim": 24, "decay": [0.5, 0.9, 0.99]},
+             "mlp": {"kind": "moe", "expert": {"ff": 48}, "shared": {"ff": 64}, "router": {"experts": 6, "top": 2}}},
+            {"type": "parallel", "mixer": {
+                "left": {"dim": 24, "vdim": 24, "heads": 4, "kv_heads": 2, "mask": {"size": 20, "pool": 5}, "scale": 0.2,
+                         "softcap": 30.0, "rot": {"base": 10000.0, "dims": 16,
+                                                  "scaling": {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}}},
+                "right": {"dim": 16, "vdim": 40, "heads": 2, "tau": 8.0}},
+             "mlp": {"kind": "moe", "expert": {"ff": 48}, "shared": None, "router": {"experts": 5, "top": 3}}},
+            {"type": "lightning", "mixer": {"heads": 2, "dim": 24, "vdim": 16, "decay": [0.7, 0.95]}, "mlp": None},
+            {"type": "parallel", "mixer": {
+                "left": {"dim": 16, "vdim": 16, "heads": 3, "kv_heads": 1, "mask": {"size": 9, "pool": 4}, "scale": 0.3,
+                         "softcap": 20.0, "rot": {"base": 500.0, "dims": 8}},
+                "right": {"dim": 24, "vdim": 16, "heads": 3, "tau": 4.0}},
+             "mlp": {"kind": "moe", "expert": {"ff": 32}, "shared": {"ff": 32}, "router": {"experts": 4, "top": 1}}},
+        ]}, name="tiny-fekizen"),
     "tiny-gpt2": ModelConfig(
         name="tiny-gpt2", arch="gpt2", vocab_size=512, hidden_size=128,
         intermediate_size=512, num_layers=4, num_heads=2, num_kv_heads=2, head_dim=64,

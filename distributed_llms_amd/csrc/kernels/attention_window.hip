@@ -4,7 +4,13 @@
 // query head h reads K/V head h / (H / G), a query at position p sees the keys j of its sequence with
 // 0 <= p - j < window and, with `chunk` > 0, floor(j / chunk) = floor(p / chunk) (attention inside fixed
 // chunks of positions); `sinks` (float32 [H], or null) adds exp(sink_h) to head h's softmax denominator
-// (a learned per-head logit that takes part in the normalisation only).  Scores, softmax weights and the weighted sum are float32; T is the storage
+// (a learned per-head logit that takes part in the normalisation only).  `softcap` > 0 turns every scaled
+// score s into softcap tanh(s / softcap).  Averaged caches kp [NB, G, PB, D] / vp [NB, G, Dv, PB] with `pool` > 0
+// (the K/V layouts with PB entries per block, a power of two >= 8, behind the same block table): beside its
+// window a query at position p also sees entries b < npool(p) = floor(max(p - window + 1, 0) / pool) -- one
+// mean key and value per block of `pool` positions that lies wholly before the window -- in the same softmax;
+// every kernel visits those entries first (32-entry tiles from entry 0), then the window's tokens.
+// Scores, softmax weights and the weighted sum are float32; T is the storage
 // type (bf16 or float).  Head sizes, window and block size are runtime values.
 //
 //   window_attn_row_kernel   one workgroup per (query token, head): keys in tiles of 256, one key per
@@ -35,6 +41,18 @@ __device__ __forceinline__ int win_lo(int pos, int window, int chunk) {
   int lo = max(0, pos - window + 1);
   if (chunk > 0) lo = max(lo, pos - pos % chunk);
   return lo;
+}
+
+// Averaged entries a query at `pos` sees: the blocks of `pool` positions that end at or before pos - window.
+__device__ __forceinline__ int win_npool(int pos, int window, int pool) {
+  return pool > 0 ? max(pos - window + 1, 0) / pool : 0;
+}
+
+// softcap tanh(s / softcap) from exp2 and a reciprocal (the matrix-core kernels; the row kernel, which is
+// the float32 path, calls tanhf): tanh(x) = 1 - 2 / (e^(2x) + 1), exact at both ends (e -> inf, e -> 0)
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 
 constexpr int kWinTile = 256;     // keys per tile = threads per workgroup
@@ -87,7 +105,8 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
     void* __restrict__ out_, const void* __restrict__ q_, const void* __restrict__ k_cache_,
     const void* __restrict__ v_cache_, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int t0, int H, int G, int D, int Dv,
-    int bs, int window, int chunk, float scale, const float* __restrict__ sinks) {
+    int bs, int window, int chunk, float scale, const float* __restrict__ sinks, float softcap,
+    const void* __restrict__ kp_, const void* __restrict__ vp_, int pool, int pbs) {
   extern __shared__ float lds[];
   float* qs = lds;                       // [D]
   float* p = qs + D;                     // [kWinTile]
@@ -99,8 +118,6 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
   const int pos = positions[t], b = tok_seq[t];
   const int lo = win_lo(pos, window, chunk);
   const T* q = (const T*)q_ + ((size_t)t * H + h) * D;
-  const T* kc = (const T*)k_cache_;
-  const T* vc = (const T*)v_cache_;
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   for (int d = tid; d < D; d += kWinTile) qs[d] = wld(q + d);
   // P.V layout: thread = (channel e of ew, key subgroup sub of nsub); channels beyond ew loop
@@ -112,37 +129,44 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
   for (int i = 0; i < kWinMaxAcc; ++i) acc[i] = 0.f;
   float m = -INFINITY, l = 0.f;
   __syncthreads();
-  for (int k0 = lo; k0 <= pos; k0 += kWinTile) {
-    const int j = k0 + tid;
-    float s = -INFINITY;
-    if (j <= pos) {
-      const int blk = bt[j / bs];
-      const int row = (blk * G + g) * bs + (j % bs);
-      rows[tid] = row;                                      // K row; V element (e) at ((row / bs) * Dv + e) * bs + row % bs
-      s = dot_row<T>(qs, kc + (size_t)row * D, D) * scale;
-    }
-    const float m_new = fmaxf(m, block_max(s, red));
-    const float pj = j <= pos ? expf(s - m_new) : 0.f;
-    p[tid] = pj;
-    const float psum = block_sum(pj, red);      // ends with a barrier: p and rows are visible
-    const float corr = expf(m - m_new);         // 0 at the first tile (m = -inf)
-    l = l * corr + psum;
-    m = m_new;
-    const int nk = min(kWinTile, pos + 1 - k0);
-#pragma unroll
-    for (int i = 0; i < kWinMaxAcc; ++i) {
-      const int e = e0 + i * ew;
-      if (sub < nsub && e < Dv) {
-        float a = acc[i] * corr;
-        for (int k = sub; k < nk; k += nsub) {
-          const int row = rows[k], hb = row / bs;
-          a = fmaf(p[k], wld(vc + ((size_t)hb * Dv + e) * bs + (row - hb * bs)), a);
-        }
-        acc[i] = a;
+  // keys first .. last (all visible) of a cache pair with `cbs` keys per block
+  auto run = [&](const T* kc, const T* vc, int cbs, int first, int last) {
+    for (int k0 = first; k0 <= last; k0 += kWinTile) {
+      const int j = k0 + tid;
+      float s = -INFINITY;
+      if (j <= last) {
+        const int blk = bt[j / cbs];
+        const int row = (blk * G + g) * cbs + (j % cbs);
+        rows[tid] = row;                                    // K row; V element (e) at ((row / cbs) * Dv + e) * cbs + row % cbs
+        s = dot_row<T>(qs, kc + (size_t)row * D, D) * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       }
+      const float m_new = fmaxf(m, block_max(s, red));
+      const float pj = j <= last ? expf(s - m_new) : 0.f;
+      p[tid] = pj;
+      const float psum = block_sum(pj, red);      // ends with a barrier: p and rows are visible
+      const float corr = expf(m - m_new);         // 0 at the first tile (m = -inf)
+      l = l * corr + psum;
+      m = m_new;
+      const int nk = min(kWinTile, last + 1 - k0);
+#pragma unroll
+      for (int i = 0; i < kWinMaxAcc; ++i) {
+        const int e = e0 + i * ew;
+        if (sub < nsub && e < Dv) {
+          float a = acc[i] * corr;
+          for (int k = sub; k < nk; k += nsub) {
+            const int row = rows[k], hb = row / cbs;
+            a = fmaf(p[k], wld(vc + ((size_t)hb * Dv + e) * cbs + (row - hb * cbs)), a);
+          }
+          acc[i] = a;
+        }
+      }
+      __syncthreads();                            // before the next tile overwrites p and rows
     }
-    __syncthreads();                            // before the next tile overwrites p and rows
-  }
+  };
+  const int np = win_npool(pos, window, pool);
+  if (np > 0) run((const T*)kp_, (const T*)vp_, pbs, 0, np - 1);
+  run((const T*)k_cache_, (const T*)v_cache_, bs, lo, pos);
   // a sink adds exp(sink) to the denominator; nothing is attended to through it
   float fin = 1.0f / l;
   if (sinks) {
@@ -172,8 +196,10 @@ static size_t win_row_lds(int D, int Dv) {
 
 static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t positions, uintptr_t tok_seq, int t0, int rows, int H, int G, int D,
-                        int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int f32, uintptr_t stream) {
+                        int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, float softcap, uintptr_t kp,
+                        uintptr_t vp, int pool, int pbs, int f32, uintptr_t stream) {
   DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0 && Dv <= kWinTile * kWinMaxAcc, "window attention heads");
+  DLLM_HOST_CHECK(pool == 0 || (pool > 0 && kp && vp && pbs > 0 && chunk == 0), "window attention averaged caches");
   DLLM_HOST_CHECK(bs > 0 && window >= 1 && chunk >= 0 && max_blocks > 0 && H <= 65535, "window attention sizes");
   const size_t lds = win_row_lds(D, Dv);
   DLLM_HOST_CHECK(lds <= 64 * 1024, "window attention head size");
@@ -181,16 +207,16 @@ static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
     hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_row_kernel<float>), dim3(rows, H), dim3(kWinTile), lds,
                        (hipStream_t)stream, (void*)out, (const void*)q, (const void*)k_cache, (const void*)v_cache,
                        (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, t0,
-                       H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks);
+                       H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks, softcap, (const void*)kp, (const void*)vp,
+                       pool, pbs);
   else
     hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_row_kernel<bf16>), dim3(rows, H), dim3(kWinTile), lds,
                        (hipStream_t)stream, (void*)out, (const void*)q, (const void*)k_cache, (const void*)v_cache,
                        (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, t0,
-                       H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks);
+                       H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks, softcap, (const void*)kp, (const void*)vp,
+                       pool, pbs);
   DLLM_HIP_CHECK(hipGetLastError());
 }
-
-
 
 // Softmax weights for the matrix cores without giving up their float32 value: e = hi + lo with hi the
 // upper 16 bits of e (a bf16 by truncation), lo = e - hi (exact in float32) cut to bf16 the same way;
@@ -226,7 +252,8 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int nseq, int nqt, int H, int G,
-    int D, int Dv, int bs, int window, int chunk, float scale, const float* __restrict__ sinks, int sub) {
+    int D, int Dv, int bs, int window, int chunk, float scale, const float* __restrict__ sinks, int sub, float softcap,
+    const bf16* __restrict__ kp_cache, const bf16* __restrict__ vp_cache, int pool, int pbs) {
   constexpr int kQT = QT, kTQ = 64 * QT;
   constexpr int DP = 32 * NQK, KROW = DP + kPad, VROW = kTK + kPad;
   constexpr int KPT = (kTK * (DP / 8) + 255) / 256, VPT = (16 * NDV * (kTK / 8) + 255) / 256;   // 16-byte pieces per thread
@@ -286,10 +313,14 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   float m[kQT], l[kQT];
 #pragma unroll
   for (int c2 = 0; c2 < kQT; ++c2) m[c2] = -INFINITY, l[c2] = 0.f;
-  const int last_pos = start + min(q0 + kTQ, n) - 1;                   // newest key any query of the tile sees
-  const int first_pos = win_lo(start + q0, window, chunk);             // oldest
   const int d8 = D >> 3;
   const float sc2 = scale * kLog2e;
+  const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap * kLog2e;   // capped scores in log2 units
+  // the cache pair, block size and key range of the phase that runs: averaged entries first, then tokens
+  const bf16* ck = k_cache;
+  const bf16* cv = v_cache;
+  int cbs = bs, cbsh = bsh, last_pos = 0;
+  int lo_q[kQT], hi_q[kQT];                                            // keys this lane's queries see in the phase
   bf16x8 kreg[KPT], vreg[VPT];
   // this thread's 16-byte pieces of a tile: K piece r = (key kj[r], columns 8 kc[r] ..), V piece r =
   // (channel vch[r], keys 8 vc[r] ..); the same for every tile
@@ -312,8 +343,8 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
       if (kj[r] >= 0) {
         const int j = kj[r], c = kc[r];
         const int kp = min(k0 + j, last_pos);
-        const size_t row = ((size_t)bt[kp >> bsh] * G + g) * bs + (kp & (bs - 1));
-        kreg[r] = *reinterpret_cast<const bf16x8*>(k_cache + row * D + 8 * c);
+        const size_t row = ((size_t)bt[kp >> cbsh] * G + g) * cbs + (kp & (cbs - 1));
+        kreg[r] = *reinterpret_cast<const bf16x8*>(ck + row * D + 8 * c);
       }
     }
 #pragma unroll
@@ -321,8 +352,8 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
       if (vch[r] >= 0) {
         const int ch = vch[r], c = vc[r];
         const int kp = min(k0 + 8 * c, last_pos & ~7);     // 8 keys of one block (bs % 8 == 0)
-        const size_t at = (((size_t)bt[kp >> bsh] * G + g) * Dv + ch) * bs + (kp & (bs - 1));
-        vreg[r] = *reinterpret_cast<const bf16x8*>(v_cache + at);
+        const size_t at = (((size_t)bt[kp >> cbsh] * G + g) * Dv + ch) * cbs + (kp & (cbs - 1));
+        vreg[r] = *reinterpret_cast<const bf16x8*>(cv + at);
       }
     }
   };
@@ -334,14 +365,11 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     for (int r = 0; r < VPT; ++r)
       if (vch[r] >= 0) *reinterpret_cast<bf16x8*>(vs + vch[r] * VROW + 8 * vc[r]) = vreg[r];
   };
-  // keys the wave's queries see: [wlo, whi]
+  // One phase: key tiles from `kfirst` (32-aligned) to last_pos; the wave's queries see keys [wlo, whi], and a
+  // tile inside [full_lo, full_hi] is seen whole by every query of the wave (no mask).
   const int wq0 = q0 + wave * 16 * kQT;
-  const int whi = start + min(wq0 + 16 * kQT - 1, n - 1), wlo = win_lo(start + wq0, window, chunk);
-  // a tile whose keys every query of the wave sees needs no mask: all keys <= the wave's first query's
-  // position and inside the window of its last one
-  const int full_hi = start + wq0, full_lo = win_lo(whi, window, chunk);
   const bool wave_full = wq0 + 16 * kQT <= n;
-  const int kfirst = first_pos & ~(kTK - 1);
+  auto run = [&](int kfirst, int wlo, int whi, int full_lo, int full_hi) {
   fetch(kfirst);
   for (int k0 = kfirst; k0 <= last_pos; k0 += kTK) {
     __syncthreads();                       // every wave is done with the previous tile
@@ -370,19 +398,20 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
       for (int c2 = 0; c2 < kQT; ++c2) {
         float p[8];
         float cm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float raw = i < 4 ? s0[c2][i] : s1[c2][i - 4];
+          p[i] = softcap > 0.f ? fast_tanh(raw * cap_in) * cap_out : raw * sc2;      // wave-uniform choice
+        }
         if (nomask) {                                      // wave-uniform: no per-element mask work
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            p[i] = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
-            cm = fmaxf(cm, p[i]);
-          }
+          for (int i = 0; i < 8; ++i) cm = fmaxf(cm, p[i]);
         } else {
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             const int kp = k0 + 8 * grp + i;
-            const float sv = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
-            const bool ok = qok[c2] && kp <= qpos[c2] && kp >= qlo[c2];
-            p[i] = ok ? sv : -INFINITY;
+            const bool ok = qok[c2] && kp <= hi_q[c2] && kp >= lo_q[c2];
+            p[i] = ok ? p[i] : -INFINITY;
             cm = fmaxf(cm, p[i]);
           }
         }
@@ -420,6 +449,29 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
       }
     }
   }
+  };
+  const int tile_last = start + min(q0 + kTQ, n) - 1;                  // position of the tile's last query
+  const int wave_last = start + min(wq0 + 16 * kQT - 1, n - 1);        // of the wave's last query
+  // ---- phase 1: the averaged entries (entry indices are the keys): query at p sees [0, npool(p) - 1]
+  const int np_tile = win_npool(tile_last, window, pool);
+  if (np_tile > 0) {                                                   // uniform over the workgroup
+    ck = kp_cache, cv = vp_cache, cbs = pbs, cbsh = __ffs(pbs) - 1, last_pos = np_tile - 1;
+#pragma unroll
+    for (int c2 = 0; c2 < kQT; ++c2) lo_q[c2] = 0, hi_q[c2] = win_npool(qpos[c2], window, pool) - 1;
+    run(0, 0, win_npool(wave_last, window, pool) - 1, 0, win_npool(start + wq0, window, pool) - 1);
+    __syncthreads();                                                   // before the next phase's first fetch lands in LDS
+  }
+  // ---- phase 2: the tokens of the window
+  {
+    ck = k_cache, cv = v_cache, cbs = bs, cbsh = bsh, last_pos = tile_last;
+#pragma unroll
+    for (int c2 = 0; c2 < kQT; ++c2) lo_q[c2] = qlo[c2], hi_q[c2] = qpos[c2];
+    const int first_pos = win_lo(start + q0, window, chunk);           // oldest key any query of the tile sees
+    // keys the wave's queries see: [wlo, whi]; a tile whose keys every query of the wave sees needs no mask:
+    // all keys <= the wave's first query's position and inside the window of its last one
+    run(first_pos & ~(kTK - 1), win_lo(start + wq0, window, chunk), wave_last, win_lo(wave_last, window, chunk),
+        start + wq0);
+  }
   // O^T accumulator: lane (col, grp) holds channels 16 dt + 4 grp + (0..3) of its query
 #pragma unroll
   for (int c2 = 0; c2 < kQT; ++c2) {
@@ -446,8 +498,8 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
 template <int NQK, int NDV, int QT>
 static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t cu, uintptr_t positions, int seq0, int nseq, int max_q_len, int H,
-                        int G, int D, int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks,
-                        uintptr_t stream) {
+                        int G, int D, int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, float softcap,
+                        uintptr_t kp, uintptr_t vp, int pool, int pbs, uintptr_t stream) {
   constexpr int kTQ = 64 * QT;
   const int nqt = (max_q_len + kTQ - 1) / kTQ;
   const int pairs = nseq * G, per_pair = nqt * (H / G);
@@ -457,7 +509,8 @@ static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
   hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV, QT>), dim3((unsigned)(per_xcd * 8)),
                      dim3(256), 0, (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
                      (const bf16*)v_cache, (const int32_t*)block_tables, max_blocks, (const int32_t*)cu,
-                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks, sub);
+                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, chunk, scale, (const float*)sinks, sub,
+                     softcap, (const bf16*)kp, (const bf16*)vp, pool, pbs);
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
@@ -475,7 +528,8 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int H, int G, int D, int Dv, int bs,
-    int window, int chunk, float scale, const float* __restrict__ sinks, int hpw, int splits, float* __restrict__ ws) {
+    int window, int chunk, float scale, const float* __restrict__ sinks, int hpw, int splits, float* __restrict__ ws,
+    float softcap, const bf16* __restrict__ kp_cache, const bf16* __restrict__ vp_cache, int pool, int pbs) {
   constexpr int DVP = 16 * NDV;
   __shared__ float so[kDW][16][DVP + 1];
   __shared__ float sml[kDW][2][16];
@@ -509,11 +563,20 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   float m = -INFINITY, l = 0.f;
   // keys of this lane's A rows inside a tile: first half row col -> key 8 (col / 4) + col % 4, second half + 4
   const int jr = 8 * (col >> 2) + (col & 3);
+  // The row's tiles of 32 keys: first the averaged entries (tiles 0 .. ptile - 1 over entries [0, np - 1] of
+  // the averaged caches), then the window's tokens (tiles from the 32-aligned k00 over positions [lo, pos]).
+  const int np = win_npool(pos, window, pool), ptile = (np + 31) >> 5;
+  const int pbsh = pool > 0 ? __ffs(pbs) - 1 : 0;
+  const int k00 = lo & ~31, ntile = ptile + ((pos - k00) >> 5) + 1;
   bf16x8 ka[NQK], kb[NQK];
-  auto load_k = [&](int k0) {
-    const int j1 = min(k0 + jr, pos), j2 = min(k0 + jr + 4, pos);
-    const bf16* r1 = k_cache + (((size_t)bt[j1 >> bsh] * G + g) * bs + (j1 & (bs - 1))) * D;
-    const bf16* r2 = k_cache + (((size_t)bt[j2 >> bsh] * G + g) * bs + (j2 & (bs - 1))) * D;
+  auto load_k = [&](int ti) {
+    const bool pooled = ti < ptile;
+    const int k0 = pooled ? 32 * ti : k00 + 32 * (ti - ptile), hi = pooled ? np - 1 : pos;
+    const bf16* kc = pooled ? kp_cache : k_cache;
+    const int cb = pooled ? pbs : bs, sh = pooled ? pbsh : bsh;
+    const int j1 = min(k0 + jr, hi), j2 = min(k0 + jr + 4, hi);
+    const bf16* r1 = kc + (((size_t)bt[j1 >> sh] * G + g) * cb + (j1 & (cb - 1))) * D;
+    const bf16* r2 = kc + (((size_t)bt[j2 >> sh] * G + g) * cb + (j2 & (cb - 1))) * D;
 #pragma unroll
     for (int s2 = 0; s2 < NQK; ++s2) {
       const int d0 = 32 * s2 + 8 * grp;
@@ -525,23 +588,29 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
       }
     }
   };
-  // the row's 32-key tiles are cut into `splits` runs, one per workgroup along z (long contexts of few
+  // the tiles are cut into `splits` runs, one per workgroup along z (long contexts of few
   // rows: the partial results meet in window_attn_merge_kernel); inside a run, tile index mod kDW = wave
-  const int k00 = lo & ~31, ntile = ((pos - k00) >> 5) + 1, tps = (ntile + splits - 1) / splits;
-  const int kstop = k00 + 32 * min(ntile, ((int)blockIdx.z + 1) * tps);
-  const int kbeg = k00 + 32 * ((int)blockIdx.z * tps + wave);
-  if (kbeg < kstop) load_k(kbeg);
-  for (int k0 = kbeg; k0 < kstop; k0 += 32 * kDW) {
+  const int tps = (ntile + splits - 1) / splits;
+  const int tstop = min(ntile, ((int)blockIdx.z + 1) * tps);
+  const int tbeg = (int)blockIdx.z * tps + wave;
+  const float cap_in = softcap > 0.f ? scale / softcap : 0.f;
+  if (tbeg < tstop) load_k(tbeg);
+  for (int ti = tbeg; ti < tstop; ti += kDW) {
+    const bool pooled = ti < ptile;
+    const int k0 = pooled ? 32 * ti : k00 + 32 * (ti - ptile);
+    const int rlo = pooled ? 0 : lo, rhi = pooled ? np - 1 : pos;
+    const bf16* vcache = pooled ? vp_cache : v_cache;
+    const int cb = pooled ? pbs : bs, sh = pooled ? pbsh : bsh;
     // this tile's V^T pieces (8 keys from k0 + 8 grp, clamped to the last piece that exists) go out first
-    const int kp8 = min(k0 + 8 * grp, pos & ~7);
-    const bf16* vbase = v_cache + ((size_t)bt[kp8 >> bsh] * G + g) * Dv * bs + (kp8 & (bs - 1));
+    const int kp8 = min(k0 + 8 * grp, rhi & ~7);
+    const bf16* vbase = vcache + ((size_t)bt[kp8 >> sh] * G + g) * Dv * cb + (kp8 & (cb - 1));
     bf16x8 va[NDV];
 #pragma unroll
     for (int dt = 0; dt < NDV; ++dt) {
       const int ch = 16 * dt + col;
 #pragma unroll
       for (int j = 0; j < 8; ++j) va[dt][j] = (bf16)0.f;
-      if (ch < Dv) va[dt] = *reinterpret_cast<const bf16x8*>(vbase + (size_t)ch * bs);
+      if (ch < Dv) va[dt] = *reinterpret_cast<const bf16x8*>(vbase + (size_t)ch * cb);
     }
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -552,14 +621,15 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
       }
     }
     // the wave's next tile's K rows are in flight during this tile's softmax and P.V
-    if (k0 + 32 * kDW < kstop) load_k(k0 + 32 * kDW);
+    if (ti + kDW < tstop) load_k(ti + kDW);
     float p[8];
     float cm = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int kp = k0 + 8 * grp + i;
-      const float sv = (i < 4 ? s0[i] : s1[i - 4]) * scale;
-      p[i] = (kp >= lo && kp <= pos) ? sv : -INFINITY;
+      const float raw = i < 4 ? s0[i] : s1[i - 4];
+      const float sv = softcap > 0.f ? softcap * fast_tanh(raw * cap_in) : raw * scale;
+      p[i] = (kp >= rlo && kp <= rhi) ? sv : -INFINITY;
       cm = fmaxf(cm, p[i]);
     }
     cm = rows_max(cm);
@@ -653,7 +723,7 @@ template <int NQK, int NDV>
 static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                           int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
                           int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int splits, uintptr_t ws,
-                          uintptr_t stream) {
+                          float softcap, uintptr_t kp, uintptr_t vp, int pool, int pbs, uintptr_t stream) {
   // heads per workgroup: 16 (all MFMA columns) when rows x K/V heads x key runs fill the chip, else halved
   // until about half the CUs have a workgroup -- the keys are re-read from L2, the columns left idle cost
   // nothing.  Key runs come first: a workgroup holds a CU's registers alone, so the call takes
@@ -666,7 +736,8 @@ static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr
                      dim3(rows, G * ((R + hpw - 1) / hpw), splits), dim3(64 * kDW), 0,
                      (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
                      (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, H, G,
-                     D, Dv, bs, window, chunk, scale, (const float*)sinks, hpw, splits, (float*)ws);
+                     D, Dv, bs, window, chunk, scale, (const float*)sinks, hpw, splits, (float*)ws, softcap, (const bf16*)kp,
+                     (const bf16*)vp, pool, pbs);
   DLLM_HIP_CHECK(hipGetLastError());
   if (splits > 1) {
     hipLaunchKernelGGL(window_attn_merge_kernel, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, (bf16*)out,
@@ -677,9 +748,9 @@ static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr
 
 // bf16 with 16-byte rows and pieces goes to the matrix cores; float32 (the exact path), odd head sizes
 // and heads wider than 256 take the row kernel
-static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs) {
+static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs, int pool, int pbs) {
   return !f32 && D % 8 == 0 && Dv % 8 == 0 && bs % 8 == 0 && (bs & (bs - 1)) == 0 && D <= 256 && Dv <= 256 && G > 0 &&
-         H % G == 0;
+         H % G == 0 && (pool == 0 || (pbs % 8 == 0 && (pbs & (pbs - 1)) == 0));
 }
 
 // Decode rows: tokens [0, rows) are one-token sequences.  `splits` > 1 with `ws` (float32
@@ -688,13 +759,14 @@ static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs) {
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
                            int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int splits, uintptr_t ws,
-                           int f32, uintptr_t stream) {
+                           float softcap, uintptr_t kp, uintptr_t vp, int pool, int pbs, int f32, uintptr_t stream) {
   if (rows <= 0) return;
-  if (win_mfma_ok(f32, H, G, D, Dv, bs) && (long)G * ((H / G + 1) / 2) <= 65535) {
+  if (win_mfma_ok(f32, H, G, D, Dv, bs, pool, pbs) && (long)G * ((H / G + 1) / 2) <= 65535) {
     DLLM_HOST_CHECK(window >= 1 && chunk >= 0 && max_blocks > 0, "window attention sizes");
+    DLLM_HOST_CHECK(pool == 0 || (pool > 0 && kp && vp && chunk == 0), "window attention averaged caches");
 #define WIN_DEC(NQK, NDV)                                                                                       \
   launch_decode<NQK, NDV>(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, rows, H, G, D, Dv, \
-                          bs, window, chunk, scale, sinks, splits, ws, stream)
+                          bs, window, chunk, scale, sinks, splits, ws, softcap, kp, vp, pool, pbs, stream)
     if (D <= 64 && Dv <= 64) WIN_DEC(2, 4);
     else if (D <= 128 && Dv <= 128) WIN_DEC(4, 8);
     else WIN_DEC(8, 16);
@@ -702,23 +774,25 @@ void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintpt
     return;
   }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, 0, rows, H, G, D, Dv, bs, window,
-              chunk, scale, sinks, f32, stream);
+              chunk, scale, sinks, softcap, kp, vp, pool, pbs, f32, stream);
 }
 
 // Prompt chunks: tokens [t0 .. tokens) of sequences [seq0, seqs).
 void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                             int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
                             int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, int chunk,
-                            float scale, uintptr_t sinks, int f32, uintptr_t stream) {
+                            float scale, uintptr_t sinks, float softcap, uintptr_t kp, uintptr_t vp, int pool, int pbs,
+                            int f32, uintptr_t stream) {
   // tokens of the decode rows come first: one per sequence before seq0
   const int t0 = seq0;
   if (tokens <= t0) return;
-  if (win_mfma_ok(f32, H, G, D, Dv, bs) && seqs > seq0 && max_q_len > 1) {
+  if (win_mfma_ok(f32, H, G, D, Dv, bs, pool, pbs) && seqs > seq0 && max_q_len > 1) {
     DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && H <= 65535 && seqs - seq0 <= 65535, "window attention heads");
     DLLM_HOST_CHECK(bs > 0 && window >= 1 && chunk >= 0 && max_blocks > 0, "window attention sizes");
+    DLLM_HOST_CHECK(pool == 0 || (pool > 0 && kp && vp && chunk == 0), "window attention averaged caches");
 #define WIN_TILE(NQK, NDV, QT)                                                                                  \
   launch_tile<NQK, NDV, QT>(out, q, k_cache, v_cache, block_tables, max_blocks, cu, positions, seq0, seqs - seq0, \
-                            max_q_len, H, G, D, Dv, bs, window, chunk, scale, sinks, stream)
+                            max_q_len, H, G, D, Dv, bs, window, chunk, scale, sinks, softcap, kp, vp, pool, pbs, stream)
     if (D <= 64 && Dv <= 64) WIN_TILE(2, 4, 1);
     else if (D <= 128 && Dv <= 128) WIN_TILE(4, 8, 1);
     else WIN_TILE(8, 16, 2);     // wide heads: 2b-size latent attention prompts 32 x 1024 +7 %, 4 x 4096 +29 % over QT = 1
@@ -726,7 +800,7 @@ void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintp
     return;
   }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, t0, tokens - t0, H, G, D, Dv, bs,
-              window, chunk, scale, sinks, f32, stream);
+              window, chunk, scale, sinks, softcap, kp, vp, pool, pbs, f32, stream);
 }
 
 }  // namespace dllm

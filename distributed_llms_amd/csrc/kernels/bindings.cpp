@@ -64,6 +64,11 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("relu_sq", &dllm::relu_sq);
   m.def("sm_embed_norm", &dllm::sm_embed_norm);
   m.def("sm_rownorm_rope", &dllm::sm_rownorm_rope);
+  m.def("sm_stream_enter", &dllm::sm_stream_enter);
+  m.def("sm_mix_add", &dllm::sm_mix_add);
+  m.def("sm_token_shift", &dllm::sm_token_shift);
+  m.def("sm_pool_blocks", &dllm::sm_pool_blocks);
+  m.def("la_scan", &dllm::la_scan);
   m.def("dr_prep", &dllm::dr_prep);
   m.def("dr_conv_prep", &dllm::dr_conv_prep);
   m.def("sm_conv_tail", &dllm::sm_conv_tail);

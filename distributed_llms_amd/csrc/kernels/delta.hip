@@ -12,7 +12,7 @@
 //   dr_scan_kernel      the recurrence over a varlen batch: a workgroup per (sequence, head, 64 value
 //                       columns); a column's state is thread-local (split over 4 lanes along dim), so a
 //                       step costs no exchange besides two 4-lane sums
-//   dr_out_norm_kernel  per (token, head): o / rms(o) * w * silu(gate)
+//   dr_out_norm_kernel  per (token, head): o / rms(o) * w * silu(gate) (or sigmoid(gate))
 #include <math.h>
 
 #include "common.h"
@@ -327,7 +327,7 @@ template <typename T>
 __global__ void __launch_bounds__(64) dr_out_norm_kernel(void* __restrict__ y_, long ldy, const float* __restrict__ o,
                                                          const void* __restrict__ gate_, long ldg, int gcol,
                                                          const void* __restrict__ w_, int H, int vdim, float eps,
-                                                         float out_scale) {
+                                                         float out_scale, int gate_sig) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* row = o + ((size_t)t * H + h) * vdim;
   const T* gate = (const T*)gate_ + (size_t)t * ldg + gcol + (size_t)h * vdim;
@@ -339,7 +339,7 @@ __global__ void __launch_bounds__(64) dr_out_norm_kernel(void* __restrict__ y_, 
   const float inv = out_scale / sqrtf(ss / (float)vdim + eps);
   for (int e = lane; e < vdim; e += 64) {
     const float z = ldf(gate + e);
-    stf(y + e, row[e] * inv * ldf(w + e) * (z * dr_sigmoid(z)));
+    stf(y + e, row[e] * inv * ldf(w + e) * (gate_sig ? dr_sigmoid(z) : z * dr_sigmoid(z)));
   }
 }
 
@@ -348,7 +348,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) dr_out_norm_vec_kernel(void* __restrict__ y_, long ldy, const float* __restrict__ o,
                                                              const void* __restrict__ gate_, long ldg, int gcol,
                                                              const void* __restrict__ w_, long heads_total, int H,
-                                                             int vdim, float eps, float out_scale) {
+                                                             int vdim, float eps, float out_scale, int gate_sig) {
   const int lph = vdim >> 3;
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   const long th = idx / lph;
@@ -367,12 +367,12 @@ __global__ void __launch_bounds__(256) dr_out_norm_vec_kernel(void* __restrict__
   ldv<8>((const T*)gate_ + (size_t)t * ldg + gcol + (size_t)h * vdim + c, gv);
   ldv<8>((const T*)w_ + c, wv);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) xv[e] = xv[e] * inv * wv[e] * (gv[e] * dr_sigmoid(gv[e]));
+  for (int e = 0; e < 8; ++e) xv[e] = xv[e] * inv * wv[e] * (gate_sig ? dr_sigmoid(gv[e]) : gv[e] * dr_sigmoid(gv[e]));
   if (ok) stv<8>((T*)y_ + (size_t)t * ldy + (size_t)h * vdim + c, xv);
 }
 
 void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
-                 int vdim, float eps, float out_scale, int f32, uintptr_t stream) {
+                 int vdim, float eps, float out_scale, int gate_sig, int f32, uintptr_t stream) {
   if (tokens <= 0) return;
   DLLM_HOST_CHECK(H > 0 && H <= 65535 && vdim > 0 && ldy >= (long)H * vdim && ldg >= gcol + (long)H * vdim && gcol >= 0,
                   "delta rule output norm sizes");
@@ -382,11 +382,11 @@ void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, i
     const long heads_total = (long)tokens * H, lanes = heads_total * lph;
     DLLM_HOST_CHECK((lanes + 255) / 256 < (1L << 31), "delta rule output norm grid");
     SM_DISPATCH(f32, dr_out_norm_vec_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream, (void*)y, ldy,
-                (const float*)o, (const void*)gate, ldg, gcol, (const void*)w, heads_total, H, vdim, eps, out_scale);
+                (const float*)o, (const void*)gate, ldg, gcol, (const void*)w, heads_total, H, vdim, eps, out_scale, gate_sig);
     return;
   }
   SM_DISPATCH(f32, dr_out_norm_kernel, dim3(tokens, H), dim3(64), 0, stream, (void*)y, ldy, (const float*)o,
-              (const void*)gate, ldg, gcol, (const void*)w, H, vdim, eps, out_scale);
+              (const void*)gate, ldg, gcol, (const void*)w, H, vdim, eps, out_scale, gate_sig);
 }
 
 }  // namespace dllm

@@ -72,7 +72,19 @@ void paged_attention_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uint
 void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int width, int vocab, int f32,
                   uintptr_t stream);
 void sm_embed_norm(uintptr_t x, uintptr_t h, uintptr_t ids, uintptr_t table, uintptr_t w, int tokens, int width,
-                   int vocab, float eps, float offset, int f32, uintptr_t stream);
+                   int vocab, float eps, float offset, float scale, uintptr_t pos_table, uintptr_t positions,
+                   int max_pos, int f32, uintptr_t stream);
+void sm_stream_enter(uintptr_t x, uintptr_t x0, uintptr_t vec, int rows, int width, int f32, uintptr_t stream);
+void sm_mix_add(uintptr_t x, uintptr_t o, uintptr_t w1, uintptr_t o2, uintptr_t w2, uintptr_t w_next, uintptr_t h,
+                int rows, int width, float eps, float coef, int f32, uintptr_t stream);
+void sm_token_shift(uintptr_t y, uintptr_t h, uintptr_t w, uintptr_t state, uintptr_t cu, uintptr_t positions,
+                    uintptr_t tok_seq, uintptr_t slots, int tokens, int width, int f32, uintptr_t stream);
+void sm_pool_blocks(uintptr_t k_cache, uintptr_t v_cache, uintptr_t kp_cache, uintptr_t vp_cache, uintptr_t block_tables,
+                    int max_blocks, uintptr_t positions, uintptr_t tok_seq, int tokens, int G, int D, int Dv, int bs,
+                    int pb, int pool, int f32, uintptr_t stream);
+void la_scan(uintptr_t o, uintptr_t proj, long ld, int qcol, int kcol, int vcol, uintptr_t decay, uintptr_t z,
+             uintptr_t z_bias, float inv_tau, float q_scale, int silu, uintptr_t state, uintptr_t cu, uintptr_t positions,
+             uintptr_t slots, int seqs, int max_q_len, int H, int D, int Dv, int f32, uintptr_t stream);
 void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, float eps, float offset, int f32,
                  uintptr_t stream);
 void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
@@ -99,15 +111,17 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
                   uintptr_t stream);
 void sm_rownorm_rope(uintptr_t q_out, uintptr_t qkv, long ld, int col0, uintptr_t q_norm, uintptr_t k_norm,
                      uintptr_t freqs, int nrot, float eps, uintptr_t k_cache, uintptr_t v_cache, uintptr_t slot_mapping,
-                     uintptr_t positions, int tokens, int H, int G, int D, int Dv, int bs, int f32, uintptr_t stream);
+                     uintptr_t positions, int tokens, int H, int G, int D, int Dv, int bs, float mag, int v_from_k,
+                     int f32, uintptr_t stream);
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
                            int Dv, int bs, int window, int chunk, float scale, uintptr_t sinks, int splits, uintptr_t ws,
-                           int f32, uintptr_t stream);
+                           float softcap, uintptr_t kp, uintptr_t vp, int pool, int pbs, int f32, uintptr_t stream);
 void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                             int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
                             int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, int chunk,
-                            float scale, uintptr_t sinks, int f32, uintptr_t stream);
+                            float scale, uintptr_t sinks, float softcap, uintptr_t kp, uintptr_t vp, int pool, int pbs,
+                            int f32, uintptr_t stream);
 // latent attention input stage and parallel layers on a float32 stream (latent.hip)
 void lat_prep(uintptr_t cq, uintptr_t down, long ld, int q_off, int q_rank, uintptr_t qn_w, int c_off, int rank,
               uintptr_t cn_w, int r_off, int rot_dim, uintptr_t freqs, int nfreq, uintptr_t positions,
@@ -146,7 +160,7 @@ void dr_conv_prep(uintptr_t u, uintptr_t bd, uintptr_t x, long ld, int col0, int
 void dr_scan(uintptr_t o, uintptr_t u, long ld, uintptr_t bd, uintptr_t state, uintptr_t cu, uintptr_t positions,
              uintptr_t slots, int seqs, int max_q_len, int H, int G, int dim, int vdim, uintptr_t stream);
 void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
-                 int vdim, float eps, float out_scale, int f32, uintptr_t stream);
+                 int vdim, float eps, float out_scale, int gate_sig, int f32, uintptr_t stream);
 void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,
                        uintptr_t gate_logits, long gate_ld, int T, int H, int k, int f32, uintptr_t stream);
 

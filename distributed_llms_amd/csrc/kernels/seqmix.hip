@@ -38,38 +38,54 @@ void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int
 }
 
 // --------------------------------------------------------------------------- embedding + RMS norm -> f32 stream
-// x = e / sqrt(mean(e^2) + eps) * (offset + w) for e = table[id], as the float32 stream and -- when h is
-// given -- also in the activation type (the input of a first sublayer that reads the stream unnormed).
+// x = e / sqrt(mean(e^2) + eps) * (offset + w) for e = table[id] * scale (+ pos_table[position], a learned
+// vector per position, when given), as the float32 stream and -- when h is given -- also in the activation
+// type (the input of a first sublayer that reads the stream unnormed).
 template <typename T>
 __global__ void __launch_bounds__(256) sm_embed_norm_kernel(float* __restrict__ x, void* __restrict__ h_,
                                                             const int32_t* __restrict__ ids,
                                                             const void* __restrict__ table_, const void* __restrict__ w_,
-                                                            int width, int vocab, float eps, float offset) {
+                                                            int width, int vocab, float eps, float offset, float scale,
+                                                            const void* __restrict__ pos_table_,
+                                                            const int32_t* __restrict__ positions, int max_pos) {
   __shared__ float red[16];
   const T* table = (const T*)table_;
   const T* w = (const T*)w_;
   int id = ids[blockIdx.x];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + (size_t)id * width;
+  const T* prow = nullptr;
+  if (pos_table_) {
+    int p = positions[blockIdx.x];
+    p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+    prow = (const T*)pos_table_ + (size_t)p * width;
+  }
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += 256) { const float v = ldf(src + i); ss += v * v; }
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = ldf(src + i) * scale + (prow ? ldf(prow + i) : 0.f);
+    ss += v * v;
+  }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
   float* dst = x + (size_t)blockIdx.x * width;
   T* h = h_ ? (T*)h_ + (size_t)blockIdx.x * width : nullptr;
   for (int i = threadIdx.x; i < width; i += 256) {
-    const float v = ldf(src + i) * inv * (offset + ldf(w + i));
+    const float e = ldf(src + i) * scale + (prow ? ldf(prow + i) : 0.f);
+    const float v = e * inv * (offset + ldf(w + i));
     dst[i] = v;
     if (h) stf(h + i, v);
   }
 }
 
 void sm_embed_norm(uintptr_t x, uintptr_t h, uintptr_t ids, uintptr_t table, uintptr_t w, int tokens, int width,
-                   int vocab, float eps, float offset, int f32, uintptr_t stream) {
+                   int vocab, float eps, float offset, float scale, uintptr_t pos_table, uintptr_t positions,
+                   int max_pos, int f32, uintptr_t stream) {
   if (tokens <= 0) return;
-  DLLM_HOST_CHECK(width > 0 && vocab > 0 && x && w, "embed_norm arguments");
+  DLLM_HOST_CHECK(width > 0 && vocab > 0 && x && w && (!pos_table || (positions && max_pos > 0)),
+                  "embed_norm arguments");
   SM_DISPATCH(f32, sm_embed_norm_kernel, dim3(tokens), dim3(256), 0, stream, (float*)x, (void*)h, (const int32_t*)ids,
-              (const void*)table, (const void*)w, width, vocab, eps, offset);
+              (const void*)table, (const void*)w, width, vocab, eps, offset, scale, (const void*)pos_table,
+              (const int32_t*)positions, max_pos);
 }
 
 // --------------------------------------------------------------------------- RMS norm of an f32 row
@@ -193,6 +209,155 @@ void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post
   SM_DISPATCH_V(f32, width % 8 == 0, sm_post_norm_add_kernel, dim3(rows), dim3(256), 0, stream, (float*)x,
                 (const void*)o, (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult,
                 offset, (const void*)o2, s1, s2);
+}
+
+// --------------------------------------------------------------------------- entry of a looped span
+// x += x0 (a second float32 stream, when given) + vec (one row [width] of the activation type for every
+// token, when given), in place.
+template <typename T>
+__global__ void __launch_bounds__(256) sm_stream_enter_kernel(float* __restrict__ x, const float* __restrict__ x0,
+                                                              const void* __restrict__ vec_, long n, int width) {
+  const T* vec = (const T*)vec_;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+    float v = x[i];
+    if (x0) v += x0[i];
+    if (vec) v += ldf(vec + (int)(i % width));
+    x[i] = v;
+  }
+}
+
+void sm_stream_enter(uintptr_t x, uintptr_t x0, uintptr_t vec, int rows, int width, int f32, uintptr_t stream) {
+  if (rows <= 0) return;
+  DLLM_HOST_CHECK(width > 0 && x, "stream_enter arguments");
+  const long n = (long)rows * width;
+  const unsigned grid = (unsigned)std::min<long>((n + 255) / 256, 65535);
+  SM_DISPATCH(f32, sm_stream_enter_kernel, dim3(grid), dim3(256), 0, stream, (float*)x, (const float*)x0,
+              (const void*)vec, n, width);
+}
+
+// --------------------------------------------------------------------------- close of a pre-norm sublayer
+// x += coef * (f(o, w1) + f(o2, w2)) with f(o, w) = o / sqrt(mean(o^2) + eps) * w when w is given and o itself
+// otherwise (o2 null: one term): two mixer outputs are normed apart, each with its own plain weight, before
+// they are summed.  With wn: h = x / sqrt(mean(x^2) + eps) * wn, the next sublayer's input.
+template <typename T, int V>
+__global__ void __launch_bounds__(256) sm_mix_add_kernel(float* __restrict__ x, const void* __restrict__ o_,
+                                                         const void* __restrict__ w1_, const void* __restrict__ o2_,
+                                                         const void* __restrict__ w2_, const void* __restrict__ wn_,
+                                                         void* __restrict__ h_, int width, float eps, float coef) {
+  __shared__ float red[16];
+  const T* o = (const T*)o_ + (size_t)blockIdx.x * width;
+  const T* o2 = o2_ ? (const T*)o2_ + (size_t)blockIdx.x * width : nullptr;
+  const T* w1 = (const T*)w1_;
+  const T* w2 = (const T*)w2_;
+  const T* wn = (const T*)wn_;
+  float* xr = x + (size_t)blockIdx.x * width;
+  float inv1 = 1.f, inv2 = 1.f;
+  if (w1 || (o2 && w2)) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+      float v[V];
+      if (w1) {
+        ldv<V>(o + i, v);
+#pragma unroll
+        for (int j = 0; j < V; ++j) s1 += v[j] * v[j];
+      }
+      if (o2 && w2) {
+        ldv<V>(o2 + i, v);
+#pragma unroll
+        for (int j = 0; j < V; ++j) s2 += v[j] * v[j];
+      }
+    }
+    if (w1) inv1 = 1.0f / sqrtf(block_sum(s1, red) / (float)width + eps);
+    if (o2 && w2) inv2 = 1.0f / sqrtf(block_sum(s2, red) / (float)width + eps);
+  }
+  float sq = 0.f;
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+    float v[V], g[V], xv[V], y[V];
+    ldv<V>(o + i, v);
+    if (w1) {
+      ldv<V>(w1 + i, g);
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = v[j] * inv1 * g[j];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) y[j] = v[j];
+    if (o2) {
+      ldv<V>(o2 + i, v);
+      if (w2) {
+        ldv<V>(w2 + i, g);
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[j] = v[j] * inv2 * g[j];
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) y[j] += v[j];
+    }
+    ldv<V>(xr + i, xv);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      xv[j] = xv[j] + coef * y[j];
+      sq += xv[j] * xv[j];
+    }
+    stv<V>(xr + i, xv);
+  }
+  if (!wn) return;
+  sq = block_sum(sq, red);
+  const float invn = 1.0f / sqrtf(sq / (float)width + eps);
+  T* h = (T*)h_ + (size_t)blockIdx.x * width;
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {      // each lane re-reads what it wrote itself
+    float xv[V], g[V];
+    ldv<V>(xr + i, xv);
+    ldv<V>(wn + i, g);
+#pragma unroll
+    for (int j = 0; j < V; ++j) xv[j] = xv[j] * invn * g[j];
+    stv<V>(h + i, xv);
+  }
+}
+
+void sm_mix_add(uintptr_t x, uintptr_t o, uintptr_t w1, uintptr_t o2, uintptr_t w2, uintptr_t w_next, uintptr_t h,
+                int rows, int width, float eps, float coef, int f32, uintptr_t stream) {
+  if (rows <= 0) return;
+  DLLM_HOST_CHECK(width > 0 && x && o && (!w_next || h) && (!w2 || o2), "mix_add arguments");
+  SM_DISPATCH_V(f32, width % 8 == 0, sm_mix_add_kernel, dim3(rows), dim3(256), 0, stream, (float*)x, (const void*)o,
+                (const void*)w1, (const void*)o2, (const void*)w2, (const void*)w_next, (void*)h, width, eps, coef);
+}
+
+// --------------------------------------------------------------------------- token shift
+// y_t = h_t + (h_(t-1) - h_t) * w per channel, h_(t-1) the UNBLENDED previous row of the same sequence: the
+// batch row before it, for a chunk's first token the row the state slot keeps (zeros at position 0).  One
+// workgroup per token; the workgroup of a chunk's FIRST token also brings the slot up to date -- it writes
+// the chunk's last row there after it has read the old one, and nobody else touches that slot in the launch.
+template <typename T>
+__global__ void __launch_bounds__(256) sm_token_shift_kernel(void* __restrict__ y_, const void* __restrict__ h_,
+                                                             const void* __restrict__ w_, void* __restrict__ state_,
+                                                             const int32_t* __restrict__ cu,
+                                                             const int32_t* __restrict__ positions,
+                                                             const int32_t* __restrict__ tok_seq,
+                                                             const int32_t* __restrict__ slots, int width) {
+  const int t = blockIdx.x, b = tok_seq[t];
+  const int lo = cu[b], hi = cu[b + 1];
+  const T* h = (const T*)h_ + (size_t)t * width;
+  const T* w = (const T*)w_;
+  T* y = (T*)y_ + (size_t)t * width;
+  const bool first = t == lo;
+  T* st = (T*)state_ + (size_t)slots[b] * width;
+  const T* prev = first ? st : h - width;
+  const bool zero = first && positions[t] == 0;
+  const T* last = (const T*)h_ + (size_t)(hi - 1) * width;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float c = ldf(h + i), p = zero ? 0.f : ldf(prev + i);
+    stf(y + i, c + (p - c) * ldf(w + i));
+    if (first) st[i] = last[i];               // same thread read st[i] just above
+  }
+}
+
+void sm_token_shift(uintptr_t y, uintptr_t h, uintptr_t w, uintptr_t state, uintptr_t cu, uintptr_t positions,
+                    uintptr_t tok_seq, uintptr_t slots, int tokens, int width, int f32, uintptr_t stream) {
+  if (tokens <= 0) return;
+  DLLM_HOST_CHECK(width > 0 && y && h && w && state && cu && positions && tok_seq && slots && y != h,
+                  "token_shift arguments");
+  SM_DISPATCH(f32, sm_token_shift_kernel, dim3(tokens), dim3(256), 0, stream, (void*)y, (const void*)h, (const void*)w,
+              (void*)state, (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots,
+              width);
 }
 
 // --------------------------------------------------------------------------- causal convolution with state
@@ -963,37 +1128,44 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
 // --------------------------------------------------------------------------- attention input: row norm + half-split rotation + append
 // From a fused projection row [.. | q (H D) | k (G D) | v (G Dv) | ..] (row stride ld, q at column `col0`):
 // an RMS norm over the WHOLE q projection and over the whole k projection (all heads at once, plain
-// weights qw [H D] / kw [G D]), then the half-split rotation of the first 2 nrot dimensions of every head:
-// dimension i < nrot is paired with dimension i + nrot, the pair turns by float(pos) * freqs[i].  q goes to
-// q_out [T, H, D]; k and v (unchanged) are appended at slot_mapping to caches k [NB, G, BS, D] / v [NB, G, Dv, BS].
+// weights qw [H D] / kw [G D]; both null: no norm), then the half-split rotation of the first 2 nrot
+// dimensions of every head: dimension i < nrot is paired with dimension i + nrot, the pair turns by
+// float(pos) * freqs[i] (cos and sin times `mag`).  q goes to q_out [T, H, D]; k and v (unchanged) are appended
+// at slot_mapping to caches k [NB, G, BS, D] / v [NB, G, Dv, BS].  `v_from_k`: the row has no v columns and
+// the values are the k columns as projected, before norm and rotation (Dv = D).
 // One workgroup per token; norms, angles and the rotation are float32.
 template <typename T>
 __global__ void __launch_bounds__(256) sm_rownorm_rope_kernel(
     void* __restrict__ q_out_, const void* __restrict__ qkv_, long ld, int col0, const void* __restrict__ qw_,
     const void* __restrict__ kw_, const float* __restrict__ freqs, int nrot, float eps, void* __restrict__ k_cache_,
     void* __restrict__ v_cache_, const int32_t* __restrict__ slot_mapping, const int32_t* __restrict__ positions, int H,
-    int G, int D, int Dv, int bs) {
+    int G, int D, int Dv, int bs, float mag, int v_from_k) {
   __shared__ float red[16];
   extern __shared__ float csn[];                   // cos | sin of the token's nrot angles
   const int t = blockIdx.x, tid = threadIdx.x;
   const float fpos = (float)positions[t];
   for (int i = tid; i < nrot; i += 256) {
     const float ang = fpos * freqs[i];
-    csn[i] = cosf(ang);
-    csn[nrot + i] = sinf(ang);
+    csn[i] = cosf(ang) * mag;
+    csn[nrot + i] = sinf(ang) * mag;
   }
   const T* q = (const T*)qkv_ + (size_t)t * ld + col0;
   const T* k = q + (size_t)H * D;
-  const T* v = k + (size_t)G * D;
+  const T* v = v_from_k ? k : k + (size_t)G * D;
   const T* qw = (const T*)qw_;
   const T* kw = (const T*)kw_;
   const int nq = H * D, nk = G * D, nv = G * Dv;
-  float sq = 0.f, sk = 0.f;
-  for (int e = tid; e < nq; e += 256) { const float x = ldf(q + e); sq += x * x; }
-  for (int e = tid; e < nk; e += 256) { const float x = ldf(k + e); sk += x * x; }
-  sq = block_sum(sq, red);
-  sk = block_sum(sk, red);
-  const float iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
+  float iq = 1.f, ik = 1.f;
+  if (qw) {
+    float sq = 0.f, sk = 0.f;
+    for (int e = tid; e < nq; e += 256) { const float x = ldf(q + e); sq += x * x; }
+    for (int e = tid; e < nk; e += 256) { const float x = ldf(k + e); sk += x * x; }
+    sq = block_sum(sq, red);
+    sk = block_sum(sk, red);
+    iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
+  } else {
+    __syncthreads();                               // csn is complete
+  }
   const int slot = slot_mapping[t], blk = slot / bs, off = slot - blk * bs;
   T* q_out = (T*)q_out_ + (size_t)t * nq;
   T* kc = (T*)k_cache_;
@@ -1005,11 +1177,13 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_kernel(
     const T* w = isq ? qw : kw;
     const float inv = isq ? iq : ik;
     const int hd = ee / D, d = ee - hd * D;
-    float x = ldf(src + ee) * inv * ldf(w + ee);
+    float x = ldf(src + ee);
+    if (w) x = x * inv * ldf(w + ee);
     if (d < 2 * nrot) {
       const int i = d < nrot ? d : d - nrot;
       const int pe = d < nrot ? ee + nrot : ee - nrot;          // the pair's other dimension
-      const float y = ldf(src + pe) * inv * ldf(w + pe);
+      float y = ldf(src + pe);
+      if (w) y = y * inv * ldf(w + pe);
       const float cs = csn[i], sn = csn[nrot + i];
       x = d < nrot ? x * cs - y * sn : x * cs + y * sn;
     }
@@ -1030,35 +1204,41 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_vec_kernel(
     void* __restrict__ q_out_, const void* __restrict__ qkv_, long ld, int col0, const void* __restrict__ qw_,
     const void* __restrict__ kw_, const float* __restrict__ freqs, int nrot, float eps, void* __restrict__ k_cache_,
     void* __restrict__ v_cache_, const int32_t* __restrict__ slot_mapping, const int32_t* __restrict__ positions, int H,
-    int G, int D, int Dv, int bs) {
+    int G, int D, int Dv, int bs, float mag, int v_from_k) {
   __shared__ float red[32];
   extern __shared__ float csn[];                   // cos | sin of the token's nrot angles
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const float fpos = (float)positions[t];
   for (int i = tid; i < nrot; i += 256) {
     const float ang = fpos * freqs[i];
-    csn[i] = cosf(ang);
-    csn[nrot + i] = sinf(ang);
+    csn[i] = cosf(ang) * mag;
+    csn[nrot + i] = sinf(ang) * mag;
   }
   const T* q = (const T*)qkv_ + (size_t)t * ld + col0;
   const int nq = H * D, nk = G * D, nv = G * Dv;
-  const T* v = q + nq + nk;
+  const T* v = v_from_k ? q + nq : q + nq + nk;
+  const bool normed = qw_ != nullptr;
   float sq = 0.f, sk = 0.f;
-  for (int e = tid * 8; e < nq + nk; e += 2048) {
-    float x[8];
-    ldv<8>(q + e, x);
-    float a = 0.f;
+  if (normed) {
+    for (int e = tid * 8; e < nq + nk; e += 2048) {
+      float x[8];
+      ldv<8>(q + e, x);
+      float a = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a += x[i] * x[i];
-    if (e < nq) sq += a; else sk += a;
+      for (int i = 0; i < 8; ++i) a += x[i] * x[i];
+      if (e < nq) sq += a; else sk += a;
+    }
+    sq = wave_sum(sq);
+    sk = wave_sum(sk);
+    if (lane == 0) red[wid] = sq, red[4 + wid] = sk;
   }
-  sq = wave_sum(sq);
-  sk = wave_sum(sk);
-  if (lane == 0) red[wid] = sq, red[4 + wid] = sk;
   __syncthreads();                                 // also: csn is complete
-  sq = red[0] + red[1] + red[2] + red[3];
-  sk = red[4] + red[5] + red[6] + red[7];
-  const float iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
+  float iq = 1.f, ik = 1.f;
+  if (normed) {
+    sq = red[0] + red[1] + red[2] + red[3];
+    sk = red[4] + red[5] + red[6] + red[7];
+    iq = 1.0f / sqrtf(sq / (float)nq + eps), ik = 1.0f / sqrtf(sk / (float)nk + eps);
+  }
   const int slot = slot_mapping[t], blk = slot / bs, off = slot - blk * bs;
   T* q_out = (T*)q_out_ + (size_t)t * nq;
   T* kc = (T*)k_cache_;
@@ -1071,19 +1251,25 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_vec_kernel(
     const int hd = ee / D, d = ee - hd * D;
     float x[8], g[8];
     ldv<8>(q + e, x);
-    ldv<8>(w, g);
+    if (normed) {
+      ldv<8>(w, g);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[i] *= inv * g[i];
+      for (int i = 0; i < 8; ++i) x[i] *= inv * g[i];
+    }
     if (d < 2 * nrot) {
       const bool first = d < nrot;
       const int po = first ? nrot : -nrot, i0 = first ? d : d - nrot;
       float y[8], gy[8];
       ldv<8>(q + e + po, y);
-      ldv<8>(w + po, gy);
+      if (normed) {
+        ldv<8>(w + po, gy);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] *= inv * gy[i];
+      }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const float yy = y[i] * inv * gy[i], cs = csn[i0 + i], sn = csn[nrot + i0 + i];
-        x[i] = first ? x[i] * cs - yy * sn : x[i] * cs + yy * sn;
+        const float cs = csn[i0 + i], sn = csn[nrot + i0 + i];
+        x[i] = first ? x[i] * cs - y[i] * sn : x[i] * cs + y[i] * sn;
       }
     }
     if (isq) stv<8>(q_out + ee, x);
@@ -1097,23 +1283,74 @@ __global__ void __launch_bounds__(256) sm_rownorm_rope_vec_kernel(
 
 void sm_rownorm_rope(uintptr_t q_out, uintptr_t qkv, long ld, int col0, uintptr_t q_norm, uintptr_t k_norm,
                      uintptr_t freqs, int nrot, float eps, uintptr_t k_cache, uintptr_t v_cache, uintptr_t slot_mapping,
-                     uintptr_t positions, int tokens, int H, int G, int D, int Dv, int bs, int f32, uintptr_t stream) {
+                     uintptr_t positions, int tokens, int H, int G, int D, int Dv, int bs, float mag, int v_from_k,
+                     int f32, uintptr_t stream) {
   if (tokens <= 0) return;
   DLLM_HOST_CHECK(H > 0 && G > 0 && D > 0 && Dv > 0 && bs > 0 && nrot >= 0 && 2 * nrot <= D && col0 >= 0 &&
-                      ld >= col0 + (long)H * D + (long)G * (D + Dv),
+                      ld >= col0 + (long)H * D + (long)G * D + (v_from_k ? 0 : (long)G * Dv) && (!v_from_k || Dv == D),
                   "rownorm_rope sizes");
-  DLLM_HOST_CHECK(q_out && k_cache && v_cache && q_norm && k_norm && (nrot == 0 || freqs), "rownorm_rope arguments");
+  DLLM_HOST_CHECK(q_out && k_cache && v_cache && (!q_norm == !k_norm) && (nrot == 0 || freqs), "rownorm_rope arguments");
   const int esz = f32 ? 4 : 2;
   if (D % 8 == 0 && nrot % 8 == 0 && ld % 8 == 0 && col0 % 8 == 0 && qkv % (8 * esz) == 0 && q_norm % (8 * esz) == 0 &&
       k_norm % (8 * esz) == 0 && q_out % (8 * esz) == 0 && k_cache % (8 * esz) == 0) {
     SM_DISPATCH(f32, sm_rownorm_rope_vec_kernel, dim3(tokens), dim3(256), 2 * (size_t)nrot * sizeof(float), stream,
                 (void*)q_out, (const void*)qkv, ld, col0, (const void*)q_norm, (const void*)k_norm, (const float*)freqs, nrot,
-                eps, (void*)k_cache, (void*)v_cache, (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs);
+                eps, (void*)k_cache, (void*)v_cache, (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs,
+                mag, v_from_k);
     return;
   }
   SM_DISPATCH(f32, sm_rownorm_rope_kernel, dim3(tokens), dim3(256), 2 * (size_t)nrot * sizeof(float), stream, (void*)q_out, (const void*)qkv, ld, col0,
               (const void*)q_norm, (const void*)k_norm, (const float*)freqs, nrot, eps, (void*)k_cache, (void*)v_cache,
-              (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs);
+              (const int32_t*)slot_mapping, (const int32_t*)positions, H, G, D, Dv, bs, mag, v_from_k);
+}
+
+// --------------------------------------------------------------------------- averaged blocks of old keys
+// For every token whose position p ends a block of `pool` positions (p + 1 a multiple of pool): the float32
+// mean of the block's keys and of its values AS THE CACHES HOLD THEM (k [NB, G, BS, D], v [NB, G, Dv, BS],
+// read through the sequence's block table) goes to entry b = (p + 1) / pool - 1 of the averaged caches
+// kp [NB, G, PB, D] / vp [NB, G, Dv, PB] (entry b at block b / PB of the same table, place b % PB).  One
+// workgroup per (token, K/V head); tokens that end no block leave at once.  Runs after the step's append.
+template <typename T>
+__global__ void __launch_bounds__(128) sm_pool_blocks_kernel(const void* __restrict__ k_cache_,
+                                                             const void* __restrict__ v_cache_, void* __restrict__ kp_,
+                                                             void* __restrict__ vp_,
+                                                             const int32_t* __restrict__ block_tables, int max_blocks,
+                                                             const int32_t* __restrict__ positions,
+                                                             const int32_t* __restrict__ tok_seq, int G, int D, int Dv,
+                                                             int bs, int pb, int pool) {
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int pos = positions[t];
+  if ((pos + 1) % pool) return;
+  const int b = (pos + 1) / pool - 1;
+  const int32_t* bt = block_tables + (size_t)tok_seq[t] * max_blocks;
+  const T* kc = (const T*)k_cache_;
+  const T* vc = (const T*)v_cache_;
+  const int pblk = bt[b / pb], poff = b % pb;
+  T* kp = (T*)kp_ + (((size_t)pblk * G + g) * pb + poff) * D;
+  T* vp = (T*)vp_ + ((size_t)pblk * G + g) * Dv * pb + poff;
+  const float inv = 1.0f / (float)pool;
+  for (int c = threadIdx.x; c < D + Dv; c += 128) {
+    float a = 0.f;
+    for (int j = b * pool; j < (b + 1) * pool; ++j) {
+      const int blk = bt[j / bs], off = j % bs;
+      a += c < D ? ldf(kc + (((size_t)blk * G + g) * bs + off) * D + c)
+                 : ldf(vc + (((size_t)blk * G + g) * Dv + (c - D)) * bs + off);
+    }
+    if (c < D) stf(kp + c, a * inv);
+    else stf(vp + (size_t)(c - D) * pb, a * inv);
+  }
+}
+
+void sm_pool_blocks(uintptr_t k_cache, uintptr_t v_cache, uintptr_t kp_cache, uintptr_t vp_cache, uintptr_t block_tables,
+                    int max_blocks, uintptr_t positions, uintptr_t tok_seq, int tokens, int G, int D, int Dv, int bs,
+                    int pb, int pool, int f32, uintptr_t stream) {
+  if (tokens <= 0) return;
+  DLLM_HOST_CHECK(G > 0 && G <= 65535 && D > 0 && Dv > 0 && bs > 0 && pb > 0 && pool > 0 && (long)pb * pool >= bs &&
+                      max_blocks > 0 && k_cache && v_cache && kp_cache && vp_cache,
+                  "pool_blocks arguments");
+  SM_DISPATCH(f32, sm_pool_blocks_kernel, dim3(tokens, G), dim3(128), 0, stream, (const void*)k_cache,
+              (const void*)v_cache, (void*)kp_cache, (void*)vp_cache, (const int32_t*)block_tables, max_blocks,
+              (const int32_t*)positions, (const int32_t*)tok_seq, G, D, Dv, bs, pb, pool);
 }
 
 }  // namespace dllm

@@ -11,6 +11,9 @@ def stage_class(arch: str):
     if arch == "zebutar":
         from .zebutar import ZebutarStage
         return ZebutarStage
+    if arch == "fekizen":
+        from .fekizen import FekizenStage
+        return FekizenStage
     if arch in ("llama", "mixtral", "gpt2"):
         from .stage import ModelStage
         return ModelStage

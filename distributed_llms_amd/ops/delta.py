@@ -151,22 +151,24 @@ def conv_unit_gates(proj: torch.Tensor, col0: int, conv_w: torch.Tensor, conv_st
 
 
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, gcol: int, w: torch.Tensor, eps: float,
-                    out_scale: float = 1.0) -> torch.Tensor:
-    """o [T, heads, vdim] float32 -> o / sqrt(mean(o^2) + eps) * w * silu(gate[:, gcol + h vdim + :]) *
-    out_scale as [T, heads vdim] in ``gate``'s dtype; ``w`` [vdim] is shared by the heads."""
+                    out_scale: float = 1.0, gate_act: str = "silu") -> torch.Tensor:
+    """o [T, heads, vdim] float32 -> o / sqrt(mean(o^2) + eps) * w * act(gate[:, gcol + h vdim + :]) *
+    out_scale as [T, heads vdim] in ``gate``'s dtype; ``w`` [vdim] is shared by the heads.  ``gate_act``:
+    "silu" (g sigmoid(g)) or "sigmoid"."""
     t, hh, dv = o.shape
-    if gate.shape[1] < gcol + hh * dv or w.numel() != dv:
+    if gate.shape[1] < gcol + hh * dv or w.numel() != dv or gate_act not in ("silu", "sigmoid"):
         raise ValueError("gated_head_norm: shape mismatch")
     if not o.is_cuda:
         z = gate[:, gcol:gcol + hh * dv].float().view(t, hh, dv)
-        y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float() * (z * torch.sigmoid(z)) * out_scale
+        ga = z * torch.sigmoid(z) if gate_act == "silu" else torch.sigmoid(z)
+        y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * w.float() * ga * out_scale
         return y.reshape(t, hh * dv).to(gate.dtype)
     _ck(o, "o", torch.float32)
     _ck(gate, "gate")
     _ck(w, "w", gate.dtype)
     y = torch.empty(t, hh * dv, dtype=gate.dtype, device=o.device)
     _k().dr_out_norm(y.data_ptr(), hh * dv, o.data_ptr(), gate.data_ptr(), gate.shape[1], int(gcol), w.data_ptr(), t, hh,
-                     dv, float(eps), float(out_scale), _f32flag(gate), _stream())
+                     dv, float(eps), float(out_scale), 1 if gate_act == "sigmoid" else 0, _f32flag(gate), _stream())
     return y
 
 

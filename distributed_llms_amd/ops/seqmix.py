@@ -82,21 +82,35 @@ def embedding_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 
 def embedding_norm_f32(ids: torch.Tensor, table: torch.Tensor, w: torch.Tensor, eps: float, one_plus: bool = True,
-                       rounded: bool = False):
-    """The RMS norm of the looked-up rows, rms(table[ids]) * ((1 if one_plus else 0) + w), as a float32
-    residual stream [T, W]; with ``rounded`` also in the table's dtype (the stream tensor itself when that
-    is float32): the input of a first sublayer that reads the stream unnormed."""
+                       rounded: bool = False, scale: float = 1.0, pos_table: Optional[torch.Tensor] = None,
+                       positions: Optional[torch.Tensor] = None):
+    """The RMS norm of the looked-up rows, rms(e) * ((1 if one_plus else 0) + w) with e = table[ids] * scale
+    (+ pos_table[positions]: a learned vector per position, unscaled), as a float32 residual stream [T, W];
+    with ``rounded`` also in the table's dtype (the stream tensor itself when that is float32): the input of
+    a first sublayer that reads the stream unnormed."""
+    if pos_table is not None and (positions is None or pos_table.shape[1] != table.shape[1] or pos_table.dtype != table.dtype):
+        raise ValueError("embedding_norm_f32: positions / position table mismatch")
     if not table.is_cuda:
-        x = _ref_rms(table.index_select(0, ids.long()), w, eps, 1.0 if one_plus else 0.0)
+        e = table.index_select(0, ids.long()).float() * scale
+        if pos_table is not None:
+            if int(positions.max()) >= pos_table.shape[0]:
+                raise ValueError("embedding_norm_f32: position beyond the position table")
+            e = e + pos_table.index_select(0, positions.long()).float()
+        x = _ref_rms(e, w, eps, 1.0 if one_plus else 0.0)
         return x, ((x if table.dtype == torch.float32 else x.to(table.dtype)) if rounded else None)
     _ck(ids, "ids", torch.int32)
     _ck(table, "table")
     _ck(w, "w", table.dtype)
+    if pos_table is not None:
+        _ck(pos_table, "pos_table", table.dtype)
+        _ck(positions, "positions", torch.int32)
     t, (v, width) = ids.numel(), table.shape
     x = torch.empty(t, width, dtype=torch.float32, device=table.device)
     h = torch.empty(t, width, dtype=table.dtype, device=table.device) if rounded and table.dtype != torch.float32 else None
     _k().sm_embed_norm(x.data_ptr(), _ptr(h), ids.data_ptr(), table.data_ptr(), w.data_ptr(), t, width, v, float(eps),
-                       1.0 if one_plus else 0.0, _f32flag(table), _stream())
+                       1.0 if one_plus else 0.0, float(scale), _ptr(pos_table),
+                       _ptr(positions) if pos_table is not None else 0, 0 if pos_table is None else pos_table.shape[0],
+                       _f32flag(table), _stream())
     return x, ((x if h is None else h) if rounded else None)
 
 
@@ -148,6 +162,90 @@ def post_norm_add(x: torch.Tensor, o: torch.Tensor, w_post: torch.Tensor, eps: f
                           float(eps), float(mult), off, _ptr(o2), float(scales[0]), float(scales[1]), _f32flag(o),
                           _stream())
     return x, (x if (plain_next and w_next is None and h is None) else h)
+
+
+def stream_enter(x: torch.Tensor, x0: Optional[torch.Tensor], vec: Optional[torch.Tensor]) -> torch.Tensor:
+    """The entry of a pass through a looped span of layers, in place on the float32 stream: x += x0 (a
+    second stream, e.g. the embedding output; None: nothing) + vec (one learned row [W] for every token;
+    None: nothing)."""
+    if x0 is not None and x0.shape != x.shape:
+        raise ValueError("stream_enter: stream shapes differ")
+    if vec is not None and vec.numel() != x.shape[1]:
+        raise ValueError("stream_enter: vector width")
+    if not x.is_cuda:
+        if x0 is not None:
+            x.add_(x0)
+        if vec is not None:
+            x.add_(vec.float())
+        return x
+    _ck(x, "x", torch.float32)
+    if x0 is not None:
+        _ck(x0, "x0", torch.float32)
+    if vec is not None:
+        _ck(vec, "vec")
+    _k().sm_stream_enter(x.data_ptr(), _ptr(x0), _ptr(vec), x.shape[0], x.shape[1],
+                         0 if vec is None else _f32flag(vec), _stream())
+    return x
+
+
+def mix_add(x: torch.Tensor, o: torch.Tensor, eps: float, w_o: Optional[torch.Tensor] = None,
+            o2: Optional[torch.Tensor] = None, w_o2: Optional[torch.Tensor] = None, coef: float = 1.0,
+            w_next: Optional[torch.Tensor] = None):
+    """The close of a pre-norm sublayer, fused, in place on the float32 stream:
+    ``x += coef * (f(o, w_o) + f(o2, w_o2))`` with f(o, w) = rms_norm(o) * w (plain weight) when ``w`` is given
+    and o itself otherwise (``o2`` None: one term) -- two mixers side by side are normed apart before they
+    are summed; with ``w_next`` also returns the next sublayer's input rms_norm(x) * w_next in ``o``'s dtype."""
+    if o.shape != x.shape or (o2 is not None and (o2.shape != x.shape or o2.dtype != o.dtype)):
+        raise ValueError("mix_add: o / x shape mismatch")
+    if not x.is_cuda:
+        f = lambda a, w: a.float() if w is None else _ref_rms(a, w, eps, 0.0)
+        y = f(o, w_o)
+        if o2 is not None:
+            y = y + f(o2, w_o2)
+        x.add_(coef * y)
+        return x, (None if w_next is None else _ref_rms(x, w_next, eps, 0.0).to(o.dtype))
+    _ck(x, "x", torch.float32)
+    _ck(o, "o")
+    if o2 is not None:
+        _ck(o2, "o2")
+    for n, w in (("w_o", w_o), ("w_o2", w_o2), ("w_next", w_next)):
+        if w is not None:
+            _ck(w, n, o.dtype)
+    h = torch.empty_like(o) if w_next is not None else None
+    _k().sm_mix_add(x.data_ptr(), o.data_ptr(), _ptr(w_o), _ptr(o2), _ptr(w_o2), _ptr(w_next), _ptr(h), x.shape[0],
+                    x.shape[1], float(eps), float(coef), _f32flag(o), _stream())
+    return x, h
+
+
+def token_shift(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
+    """Every channel of a token's row blended with the same channel of the token before it:
+    y_t = h_t + (h_(t-1) - h_t) * w, with h_(t-1) the UNBLENDED previous row of the same sequence -- the
+    chunk's own earlier row, the row ``state`` [slots, W] keeps across chunk borders, zeros before position
+    0.  ``state`` is brought up to date (the chunk's last row).  float32 arithmetic, ``h``'s dtype out."""
+    t, width = h.shape
+    if w.numel() != width or state.shape[1] != width or state.dtype != h.dtype:
+        raise ValueError("token_shift: shape / dtype mismatch")
+    if not h.is_cuda:
+        out = torch.empty_like(h)
+        cu, pos, slots = sb.cu.tolist(), sb.positions.tolist(), sb.state_slots.tolist()
+        for b in range(sb.num_seqs):
+            lo, hi = cu[b], cu[b + 1]
+            if hi == lo:
+                continue
+            first = state[slots[b]].float() if pos[lo] > 0 else torch.zeros(width)
+            cur = h[lo:hi].float()
+            prev = torch.cat([first[None], cur[:-1]], 0)
+            out[lo:hi] = (cur + (prev - cur) * w.float()).to(h.dtype)
+            state[slots[b]] = h[hi - 1]
+        return out
+    _ck(h, "h")
+    _ck(w, "w", h.dtype)
+    _ck(state, "state", h.dtype)
+    out = torch.empty_like(h)
+    _k().sm_token_shift(out.data_ptr(), h.data_ptr(), w.data_ptr(), state.data_ptr(), sb.cu.data_ptr(),
+                        sb.positions.data_ptr(), sb.tok_seq.data_ptr(), sb.state_slots.data_ptr(), t, width, _f32flag(h),
+                        _stream())
+    return out
 
 
 # ------------------------------------------------------------------ causal convolution with state
@@ -400,12 +498,12 @@ def rotary_frequencies(dims: int, base: float) -> torch.Tensor:
     return yarn_frequencies(dims, base, None)[0]
 
 
-def _ref_rope_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+def _ref_rope_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, mag: float = 1.0) -> torch.Tensor:
     """x [T, H, D] float32; dimension i < len(freqs) is paired with dimension i + len(freqs); the pair
-    (u, v) turns to (u cos a - v sin a, v cos a + u sin a), a = pos * f_i."""
+    (u, v) turns to (u cos a - v sin a, v cos a + u sin a), a = pos * f_i (cos and sin times ``mag``)."""
     n = freqs.numel()
     ang = pos.float()[:, None] * freqs.float()[None]
-    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    c, s = (torch.cos(ang) * mag)[:, None, :], (torch.sin(ang) * mag)[:, None, :]
     out = x.clone()
     a, b = x[..., :n], x[..., n:2 * n]
     out[..., :n] = a * c - b * s
@@ -413,43 +511,97 @@ def _ref_rope_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor) -> t
     return out
 
 
-def rownorm_rope(qkv: torch.Tensor, col0: int, q_norm: torch.Tensor, k_norm: torch.Tensor, freqs: torch.Tensor,
-                 eps: float, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
-                 positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+def rownorm_rope(qkv: torch.Tensor, col0: int, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor],
+                 freqs: torch.Tensor, eps: float, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                 positions: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, mag: float = 1.0,
+                 v_from_k: bool = False) -> torch.Tensor:
     """From columns ``col0 ..`` of a fused projection [T, .. | q (heads dim) | k (kv_heads dim) | v (kv_heads
     vdim) | ..]: an RMS norm over the WHOLE q projection and over the whole k projection (all heads at
-    once; plain weights ``q_norm`` [heads dim], ``k_norm`` [kv_heads dim]), then the half-split rotation
-    of the first 2 len(freqs) dimensions of every q and k head (dimension i paired with i + len(freqs),
-    angle position * freqs[i]), and the append of k and v (v unchanged) at ``slot_mapping`` into caches
-    k [NB, kv_heads, BS, dim] / v [NB, kv_heads, vdim, BS].  Returns q [T, heads, dim]."""
+    once; plain weights ``q_norm`` [heads dim], ``k_norm`` [kv_heads dim]; both None: no norm), then the
+    half-split rotation of the first 2 len(freqs) dimensions of every q and k head (dimension i paired
+    with i + len(freqs), angle position * freqs[i], cos and sin times ``mag``), and the append of k and v
+    (v unchanged) at ``slot_mapping`` into caches k [NB, kv_heads, BS, dim] / v [NB, kv_heads, vdim, BS].
+    ``v_from_k``: the projection has no v columns; the values are the keys as projected, BEFORE norm and
+    rotation (vdim = dim).  Returns q [T, heads, dim]."""
     t = qkv.shape[0]
     nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
-    if qkv.shape[1] < col0 + nq + nk + nv or q_norm.numel() != nq or k_norm.numel() != nk or 2 * freqs.numel() > dim:
+    normed = q_norm is not None
+    if (k_norm is not None) != normed or (v_from_k and vdim != dim) or 2 * freqs.numel() > dim:
+        raise ValueError("rownorm_rope: norm weights for both or neither; values from keys need vdim = dim")
+    if qkv.shape[1] < col0 + nq + nk + (0 if v_from_k else nv) or (normed and (q_norm.numel() != nq or k_norm.numel() != nk)):
         raise ValueError("rownorm_rope: shape mismatch")
     bs = k_cache.shape[2]
     if k_cache.shape[1:] != (kv_heads, bs, dim) or v_cache.shape[1:] != (kv_heads, vdim, bs):
         raise ValueError("rownorm_rope: cache shape")
     if not qkv.is_cuda:
-        x = qkv[:, col0:col0 + nq + nk + nv].float()
-        q = _ref_rope_half(_ref_rms(x[:, :nq], q_norm, eps, 0.0).view(t, heads, dim), positions, freqs)
-        k = _ref_rope_half(_ref_rms(x[:, nq:nq + nk], k_norm, eps, 0.0).view(t, kv_heads, dim), positions, freqs)
+        x = qkv[:, col0:col0 + nq + nk].float()
+        xq, xk = x[:, :nq], x[:, nq:]
+        if normed:
+            xq, xk = _ref_rms(xq, q_norm, eps, 0.0), _ref_rms(xk, k_norm, eps, 0.0)
+        q = _ref_rope_half(xq.reshape(t, heads, dim), positions, freqs, mag)
+        k = _ref_rope_half(xk.reshape(t, kv_heads, dim), positions, freqs, mag)
         slot = slot_mapping.long()
         k_cache[slot // bs, :, slot % bs] = k.to(k_cache.dtype)
-        v_cache[slot // bs, :, :, slot % bs] = qkv[:, col0 + nq + nk:col0 + nq + nk + nv].reshape(t, kv_heads, vdim).to(
-            v_cache.dtype)
+        v0 = col0 + nq if v_from_k else col0 + nq + nk
+        v_cache[slot // bs, :, :, slot % bs] = qkv[:, v0:v0 + nv].reshape(t, kv_heads, vdim).to(v_cache.dtype)
         return q.to(qkv.dtype)
     _ck(qkv, "qkv")
-    _ck(q_norm, "q_norm", qkv.dtype)
-    _ck(k_norm, "k_norm", qkv.dtype)
+    if normed:
+        _ck(q_norm, "q_norm", qkv.dtype)
+        _ck(k_norm, "k_norm", qkv.dtype)
     _ck(freqs, "freqs", torch.float32)
     _ck(k_cache, "k_cache", qkv.dtype)
     _ck(v_cache, "v_cache", qkv.dtype)
     q = torch.empty(t, heads, dim, dtype=qkv.dtype, device=qkv.device)
-    _k().sm_rownorm_rope(q.data_ptr(), qkv.data_ptr(), qkv.shape[1], int(col0), q_norm.data_ptr(), k_norm.data_ptr(),
+    _k().sm_rownorm_rope(q.data_ptr(), qkv.data_ptr(), qkv.shape[1], int(col0), _ptr(q_norm), _ptr(k_norm),
                          freqs.data_ptr(), freqs.numel(), float(eps), k_cache.data_ptr(), v_cache.data_ptr(),
-                         slot_mapping.data_ptr(), positions.data_ptr(), t, heads, kv_heads, dim, vdim, bs,
-                         _f32flag(qkv), _stream())
+                         slot_mapping.data_ptr(), positions.data_ptr(), t, heads, kv_heads, dim, vdim, bs, float(mag),
+                         1 if v_from_k else 0, _f32flag(qkv), _stream())
     return q
+
+
+# ------------------------------------------------------------------ averaged blocks of old keys
+def pooled_block_size(block_size: int, pool: int) -> int:
+    """Entries per cache block of the averaged-key cache: a power of two >= 8 that holds at least
+    ceil(block_size / pool) entries, so that entry b (written when position b pool + pool - 1 arrives) lies in
+    a block the sequence already owns: block floor(b / entries) <= floor((b pool + pool - 1) / block_size)."""
+    need, n = -(-block_size // pool), 8
+    while n < need:
+        n *= 2
+    return n
+
+
+def pool_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, kp_cache: torch.Tensor, vp_cache: torch.Tensor,
+                block_tables: torch.Tensor, sb: SeqBatch, pool: int) -> None:
+    """Averaged keys and values of whole blocks of ``pool`` positions: for every token of the step whose
+    position p ends a block (p + 1 a multiple of pool), the float32 mean of the block's ``pool`` keys and of
+    its values AS THE CACHES HOLD THEM goes to entry b = (p + 1) / pool - 1 of the sequence's averaged
+    caches kp [NB, G, PB, dim] / vp [NB, G, vdim, PB] (the K/V layouts with PB entries per block, behind the
+    same block table: entry b at block b // PB, place b % PB).  Run after the step's keys are appended: a
+    block's keys may come from earlier steps and from this one."""
+    g, bs, d = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    dv, pb = v_cache.shape[2], kp_cache.shape[2]
+    if pool < 1 or kp_cache.shape[1:] != (g, pb, d) or vp_cache.shape[1:] != (g, dv, pb) or pb * pool < bs:
+        raise ValueError("pool_blocks: cache shapes")
+    if not k_cache.is_cuda:
+        pos, seq = sb.positions.tolist(), sb.tok_seq.tolist()
+        for i in range(sb.num_tokens):
+            if (pos[i] + 1) % pool:
+                continue
+            b = (pos[i] + 1) // pool - 1
+            bt = block_tables[seq[i]].long()
+            idx = torch.arange(b * pool, (b + 1) * pool)
+            kk = k_cache[bt[idx // bs], :, idx % bs].float().mean(0)          # [G, d]
+            vv = v_cache[bt[idx // bs], :, :, idx % bs].float().mean(0)       # [G, dv]
+            kp_cache[bt[b // pb], :, b % pb] = kk.to(kp_cache.dtype)
+            vp_cache[bt[b // pb], :, :, b % pb] = vv.to(vp_cache.dtype)
+        return
+    for n, c in (("k_cache", k_cache), ("v_cache", v_cache), ("kp_cache", kp_cache), ("vp_cache", vp_cache)):
+        _ck(c, n, k_cache.dtype)
+    _ck(block_tables, "block_tables", torch.int32)
+    _k().sm_pool_blocks(k_cache.data_ptr(), v_cache.data_ptr(), kp_cache.data_ptr(), vp_cache.data_ptr(),
+                        block_tables.data_ptr(), block_tables.shape[1], sb.positions.data_ptr(), sb.tok_seq.data_ptr(),
+                        sb.num_tokens, g, d, dv, bs, pb, int(pool), _f32flag(k_cache), _stream())
 
 
 # ------------------------------------------------------------------ sliding-window attention
@@ -466,7 +618,8 @@ def decode_splits(rows: int, heads: int, kv_heads: int, ctx: int) -> int:
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                      sb: SeqBatch, window: int, scale: float, num_decode: Optional[int] = None,
-                     sinks: Optional[torch.Tensor] = None, max_ctx: Optional[int] = None, chunk: int = 0) -> torch.Tensor:
+                     sinks: Optional[torch.Tensor] = None, max_ctx: Optional[int] = None, chunk: int = 0,
+                     softcap: float = 0.0, pooled: Optional[tuple] = None) -> torch.Tensor:
     """Softmax attention of every query token over the keys j of its own sequence with
     0 <= p - j < window (p the query's position) and, with ``chunk`` > 0, floor(j / chunk) =
     floor(p / chunk) (attention inside fixed chunks of positions counted from position 0, wherever a
@@ -478,9 +631,21 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     logit that takes part in the normalisation only (nothing is attended to through it; it enters as it
     is, without the score scale).  ``max_ctx``: a bound on the decode
     rows' context; with few rows of long context their keys are cut into runs on separate workgroups
-    (results equal up to rounding).  Returns [T, H, vdim]."""
+    (results equal up to rounding).  ``softcap`` > 0: every scaled score s becomes softcap * tanh(s / softcap).
+    ``pooled`` = (kp_cache, vp_cache, pool): beside the tokens of its window a query at position p sees one
+    averaged key and value for every block of ``pool`` positions that lies wholly before the window -- entries
+    b < floor((p - window + 1) / pool) of the averaged caches (:func:`pool_blocks`), scored, capped and
+    normalised in the same softmax; tokens that left the window inside a block not yet complete are not
+    seen at all.  Returns [T, H, vdim]."""
     t, h, d = q.shape
     g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    kp = vp = None
+    pool, pb = 0, 1
+    if pooled is not None:
+        kp, vp, pool = pooled
+        pb = kp.shape[2]
+        if pool < 1 or chunk or kp.shape[1:] != (g, pb, d) or vp.shape[1:] != (g, dv, pb) or pb * pool < bs:
+            raise ValueError("window_attention: averaged caches do not fit (and exclude a chunk mask)")
     if not q.is_cuda:
         out = torch.empty(t, h, dv, dtype=torch.float32)
         pos, seq = sb.positions.tolist(), sb.tok_seq.tolist()
@@ -492,12 +657,19 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             blk = block_tables[seq[i]].long()[idx // bs]
             kk = k_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)     # [n, H, d]
             vv = v_cache[blk, :, :, idx % bs].float().repeat_interleave(rep, 1)
+            if pool and p - window + 1 >= pool:
+                pidx = torch.arange((p - window + 1) // pool)
+                pblk = block_tables[seq[i]].long()[pidx // pb]
+                kk = torch.cat([kp[pblk, :, pidx % pb].float().repeat_interleave(rep, 1), kk], 0)
+                vv = torch.cat([vp[pblk, :, :, pidx % pb].float().repeat_interleave(rep, 1), vv], 0)
             s = torch.einsum("hd,nhd->hn", q[i].float(), kk) * scale
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
             if sinks is not None:      # one more column in the softmax whose weight is dropped
-                p = torch.softmax(torch.cat([s, sinks.float()[:, None]], -1), -1)[:, :-1]
+                pr = torch.softmax(torch.cat([s, sinks.float()[:, None]], -1), -1)[:, :-1]
             else:
-                p = torch.softmax(s, -1)
-            out[i] = torch.einsum("hn,nhd->hd", p, vv)
+                pr = torch.softmax(s, -1)
+            out[i] = torch.einsum("hn,nhd->hd", pr, vv)
         return out.to(q.dtype)
     _ck(q, "q")
     _ck(k_cache, "k_cache", q.dtype)
@@ -509,22 +681,29 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         _ck(sinks, "sinks", torch.float32)
         if sinks.numel() != h:
             raise ValueError("window_attention: one sink per query head")
+    if pool:
+        _ck(kp, "kp_cache", q.dtype)
+        _ck(vp, "vp_cache", q.dtype)
     out = torch.empty(t, h, dv, dtype=q.dtype, device=q.device)
     nd = sb.num_seqs if num_decode is None else int(num_decode)
     f = _f32flag(q)
     if nd:       # one-token rows are the first nd tokens
         span = min(int(window), int(chunk)) if chunk > 0 else int(window)
-        splits, ws = decode_splits(nd, h, g, min(span, int(max_ctx or 0))), None
+        ctx = int(max_ctx or 0)
+        keys = min(span, ctx) + (max(0, ctx - span) // pool if pool else 0)      # window tokens + averaged entries
+        splits, ws = decode_splits(nd, h, g, keys), None
         if splits > 1 and not f:
             ws = torch.empty(nd * h * splits * (dv + 2), dtype=torch.float32, device=q.device)
         _k().sm_window_attn_decode(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                    block_tables.data_ptr(), block_tables.shape[1], sb.positions.data_ptr(),
                                    sb.tok_seq.data_ptr(), nd, h, g, d, dv, bs, int(window), int(chunk), float(scale), _ptr(sinks),
-                                   splits if ws is not None else 1, _ptr(ws), f, _stream())
+                                   splits if ws is not None else 1, _ptr(ws), float(softcap), _ptr(kp), _ptr(vp), int(pool),
+                                   int(pb), f, _stream())
     if t > nd:
         _k().sm_window_attn_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                     block_tables.data_ptr(), block_tables.shape[1], sb.cu.data_ptr(),
                                     sb.positions.data_ptr(), sb.tok_seq.data_ptr(), nd, sb.num_seqs, t, sb.max_q_len,
                                     h, g, d, dv, bs,
-                                    int(window), int(chunk), float(scale), _ptr(sinks), f, _stream())
+                                    int(window), int(chunk), float(scale), _ptr(sinks), float(softcap), _ptr(kp), _ptr(vp),
+                                    int(pool), int(pb), f, _stream())
     return out
