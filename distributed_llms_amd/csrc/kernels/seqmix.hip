@@ -1328,7 +1328,7 @@ __global__ void __launch_bounds__(128) sm_pool_blocks_kernel(const void* __restr
   const int pblk = bt[b / pb], poff = b % pb;
   T* kp = (T*)kp_ + (((size_t)pblk * G + g) * pb + poff) * D;
   T* vp = (T*)vp_ + ((size_t)pblk * G + g) * Dv * pb + poff;
-  const float inv = 1.0f / (float)pool;
+  const float fpool = (float)pool;
   for (int c = threadIdx.x; c < D + Dv; c += 128) {
     float a = 0.f;
     for (int j = b * pool; j < (b + 1) * pool; ++j) {
@@ -1336,8 +1336,8 @@ __global__ void __launch_bounds__(128) sm_pool_blocks_kernel(const void* __restr
       a += c < D ? ldf(kc + (((size_t)blk * G + g) * bs + off) * D + c)
                  : ldf(vc + (((size_t)blk * G + g) * Dv + (c - D)) * bs + off);
     }
-    if (c < D) stf(kp + c, a * inv);
-    else stf(vp + (size_t)(c - D) * pb, a * inv);
+    if (c < D) stf(kp + c, a / fpool);
+    else stf(vp + (size_t)(c - D) * pb, a / fpool);
   }
 }
 

@@ -337,7 +337,8 @@ def test_window_with_averaged_blocks_capped_scores_and_a_sink(target, shape):
         kpw = np.stack([kk[b * pool:(b + 1) * pool].float().mean(0).to(dtype).double().numpy() for b in range(nblk)])
         vpw = np.stack([vv[b * pool:(b + 1) * pool].float().mean(0).to(dtype).double().numpy() for b in range(nblk)])
         for b in range(nblk):
-            np.testing.assert_allclose(kp[table[b // pb], :, b % pb].double().cpu().numpy(), kpw[b], atol=1e-6 if dtype == torch.float32 else 1e-2)
+            np.testing.assert_allclose(kp[table[b // pb], :, b % pb].double().cpu().numpy(), kpw[b],
+                                       **(dict(rtol=1e-6, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)))
         return kc, vc, kp, vp, kpw, vpw
 
     def run(qq, caches, lo, p, decode):
@@ -542,7 +543,7 @@ def test_mixer_outputs_normed_apart_then_averaged(target, width):
     np.testing.assert_allclose(xg.cpu().numpy(), d(x) + d(o1), atol=1e-5)
     # gated norms: ``groups`` heads share w; one group = all heads normed together
     hh, dv = 3, 8
-    o = torch.from_numpy(rng.standard_normal((t, hh * dv)).astype(np.float32) * np.repeat([9.0, 1.0, 0.1], dv))
+    o = torch.from_numpy((rng.standard_normal((t, hh * dv)) * np.repeat([9.0, 1.0, 0.1], dv)).astype(np.float32))
     gate = T(rng.standard_normal((t, 5 + hh * dv)))
     w_all, w_head = T(1 + 0.3 * rng.standard_normal(hh * dv)), T(1 + 0.3 * rng.standard_normal(dv))
     y = la.gated_norm(o.to(device), gate.to(device), 5, w_all.to(device), 1e-6, groups=1, gate_act="sigmoid")
