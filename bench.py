@@ -92,7 +92,8 @@ def parse(argv=None):
                     help="--hybrid: the models to run: tudilix,llama (sliding-window attention + RG-LRU beside Llama) "
                          "or gikovik,mixtral (latent attention + grouped-choice experts beside Mixtral), or "
                          "zebutar,mixtral (chunked attention beside a gated delta rule + SwiGLU experts beside "
-                         "Mixtral), or one of them")
+                         "Mixtral), or fekizen,zebutar,mixtral (window attention with averaged blocks beside gated "
+                         "linear attention, lightning layers + SwiGLU experts, beside both), or one of them")
     return ap.parse_args(argv)
 
 

@@ -371,12 +371,51 @@ __global__ void __launch_bounds__(256) dr_out_norm_vec_kernel(void* __restrict__
   if (ok) stv<8>((T*)y_ + (size_t)t * ldy + (size_t)h * vdim + c, xv);
 }
 
+// The same for groups wider than 512 channels (one norm over many heads at once): a workgroup per (token, group),
+// 8 channels per lane and step.
+template <typename T>
+__global__ void __launch_bounds__(256) dr_out_norm_wide_kernel(void* __restrict__ y_, long ldy, const float* __restrict__ o,
+                                                              const void* __restrict__ gate_, long ldg, int gcol,
+                                                              const void* __restrict__ w_, int H, int vdim, float eps,
+                                                              float out_scale, int gate_sig) {
+  __shared__ float red[16];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* row = o + ((size_t)t * H + h) * vdim;
+  const T* gate = (const T*)gate_ + (size_t)t * ldg + gcol + (size_t)h * vdim;
+  const T* w = (const T*)w_;
+  T* y = (T*)y_ + (size_t)t * ldy + (size_t)h * vdim;
+  float ss = 0.f;
+  for (int e = threadIdx.x * 8; e < vdim; e += 2048) {
+    float xv[8];
+    ldv<8>(row + e, xv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += xv[i] * xv[i];
+  }
+  ss = block_sum(ss, red);
+  const float inv = out_scale / sqrtf(ss / (float)vdim + eps);
+  for (int e = threadIdx.x * 8; e < vdim; e += 2048) {
+    float xv[8], gv[8], wv[8];
+    ldv<8>(row + e, xv);
+    ldv<8>(gate + e, gv);
+    ldv<8>(w + e, wv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xv[i] = xv[i] * inv * wv[i] * (gate_sig ? dr_sigmoid(gv[i]) : gv[i] * dr_sigmoid(gv[i]));
+    stv<8>(y + e, xv);
+  }
+}
+
 void dr_out_norm(uintptr_t y, long ldy, uintptr_t o, uintptr_t gate, long ldg, int gcol, uintptr_t w, int tokens, int H,
                  int vdim, float eps, float out_scale, int gate_sig, int f32, uintptr_t stream) {
   if (tokens <= 0) return;
   DLLM_HOST_CHECK(H > 0 && H <= 65535 && vdim > 0 && ldy >= (long)H * vdim && ldg >= gcol + (long)H * vdim && gcol >= 0,
                   "delta rule output norm sizes");
   const int esz = f32 ? 4 : 2, lph = vdim >> 3;
+  if (vdim % 8 == 0 && vdim > 512 && ldy % 8 == 0 && ldg % 8 == 0 && gcol % 8 == 0 && y % (8 * esz) == 0 &&
+      gate % (8 * esz) == 0 && w % (8 * esz) == 0 && o % 32 == 0) {
+    SM_DISPATCH(f32, dr_out_norm_wide_kernel, dim3(tokens, H), dim3(256), 0, stream, (void*)y, ldy, (const float*)o,
+                (const void*)gate, ldg, gcol, (const void*)w, H, vdim, eps, out_scale, gate_sig);
+    return;
+  }
   if (vdim % 8 == 0 && lph <= 64 && (lph & (lph - 1)) == 0 && ldy % 8 == 0 && ldg % 8 == 0 && gcol % 8 == 0 &&
       y % (8 * esz) == 0 && gate % (8 * esz) == 0 && w % (8 * esz) == 0 && o % 32 == 0) {
     const long heads_total = (long)tokens * H, lanes = heads_total * lph;

@@ -80,8 +80,8 @@ void sm_mix_add(uintptr_t x, uintptr_t o, uintptr_t w1, uintptr_t o2, uintptr_t 
 void sm_token_shift(uintptr_t y, uintptr_t h, uintptr_t w, uintptr_t state, uintptr_t cu, uintptr_t positions,
                     uintptr_t tok_seq, uintptr_t slots, int tokens, int width, int f32, uintptr_t stream);
 void sm_pool_blocks(uintptr_t k_cache, uintptr_t v_cache, uintptr_t kp_cache, uintptr_t vp_cache, uintptr_t block_tables,
-                    int max_blocks, uintptr_t positions, uintptr_t tok_seq, int tokens, int G, int D, int Dv, int bs,
-                    int pb, int pool, int f32, uintptr_t stream);
+                    int max_blocks, uintptr_t cu, uintptr_t positions, int seqs, int max_q_len, int G, int D, int Dv,
+                    int bs, int pb, int pool, int f32, uintptr_t stream);
 void la_scan(uintptr_t o, uintptr_t proj, long ld, int qcol, int kcol, int vcol, uintptr_t decay, uintptr_t z,
              uintptr_t z_bias, float inv_tau, float q_scale, int silu, uintptr_t state, uintptr_t cu, uintptr_t positions,
              uintptr_t slots, int seqs, int max_q_len, int H, int D, int Dv, int f32, uintptr_t stream);

@@ -326,7 +326,7 @@ void sm_mix_add(uintptr_t x, uintptr_t o, uintptr_t w1, uintptr_t o2, uintptr_t 
 // batch row before it, for a chunk's first token the row the state slot keeps (zeros at position 0).  One
 // workgroup per token; the workgroup of a chunk's FIRST token also brings the slot up to date -- it writes
 // the chunk's last row there after it has read the old one, and nobody else touches that slot in the launch.
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_token_shift_kernel(void* __restrict__ y_, const void* __restrict__ h_,
                                                              const void* __restrict__ w_, void* __restrict__ state_,
                                                              const int32_t* __restrict__ cu,
@@ -343,10 +343,23 @@ __global__ void __launch_bounds__(256) sm_token_shift_kernel(void* __restrict__ 
   const T* prev = first ? st : h - width;
   const bool zero = first && positions[t] == 0;
   const T* last = (const T*)h_ + (size_t)(hi - 1) * width;
-  for (int i = threadIdx.x; i < width; i += 256) {
-    const float c = ldf(h + i), p = zero ? 0.f : ldf(prev + i);
-    stf(y + i, c + (p - c) * ldf(w + i));
-    if (first) st[i] = last[i];               // same thread read st[i] just above
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+    float c[V], p[V], g[V];
+    ldv<V>(h + i, c);
+    ldv<V>(w + i, g);
+    if (zero) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) p[j] = 0.f;
+    } else {
+      ldv<V>(prev + i, p);
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) c[j] = c[j] + (p[j] - c[j]) * g[j];
+    stv<V>(y + i, c);
+    if (first) {                                // same thread read st[i ..] just above
+      ldv<V>(last + i, p);
+      stv<V>(st + i, p);
+    }
   }
 }
 
@@ -355,9 +368,11 @@ void sm_token_shift(uintptr_t y, uintptr_t h, uintptr_t w, uintptr_t state, uint
   if (tokens <= 0) return;
   DLLM_HOST_CHECK(width > 0 && y && h && w && state && cu && positions && tok_seq && slots && y != h,
                   "token_shift arguments");
-  SM_DISPATCH(f32, sm_token_shift_kernel, dim3(tokens), dim3(256), 0, stream, (void*)y, (const void*)h, (const void*)w,
-              (void*)state, (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots,
-              width);
+  const int esz = f32 ? 4 : 2;
+  const bool vec = width % 8 == 0 && y % (8 * esz) == 0 && h % (8 * esz) == 0 && w % (8 * esz) == 0 && state % (8 * esz) == 0;
+  SM_DISPATCH_V(f32, vec, sm_token_shift_kernel, dim3(tokens), dim3(256), 0, stream, (void*)y, (const void*)h,
+                (const void*)w, (void*)state, (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq,
+                (const int32_t*)slots, width);
 }
 
 // --------------------------------------------------------------------------- causal convolution with state
@@ -1305,52 +1320,69 @@ void sm_rownorm_rope(uintptr_t q_out, uintptr_t qkv, long ld, int col0, uintptr_
 }
 
 // --------------------------------------------------------------------------- averaged blocks of old keys
-// For every token whose position p ends a block of `pool` positions (p + 1 a multiple of pool): the float32
-// mean of the block's keys and of its values AS THE CACHES HOLD THEM (k [NB, G, BS, D], v [NB, G, Dv, BS],
-// read through the sequence's block table) goes to entry b = (p + 1) / pool - 1 of the averaged caches
-// kp [NB, G, PB, D] / vp [NB, G, Dv, PB] (entry b at block b / PB of the same table, place b % PB).  One
-// workgroup per (token, K/V head); tokens that end no block leave at once.  Runs after the step's append.
-template <typename T>
+// For every block of `pool` positions whose LAST position p (p + 1 a multiple of pool) is a token of this
+// step: the float32 mean of the block's keys and of its values AS THE CACHES HOLD THEM (k [NB, G, BS, D],
+// v [NB, G, Dv, BS], read through the sequence's block table; earlier steps may have written some of them)
+// goes to entry b = (p + 1) / pool - 1 of the averaged caches kp [NB, G, PB, D] / vp [NB, G, Dv, PB] (entry b
+// at block b / PB of the same table, place b % PB).  One workgroup per (block that a chunk may complete, K/V
+// head, sequence); V consecutive key dimensions per lane.  Runs after the step's append.
+template <typename T, int V>
 __global__ void __launch_bounds__(128) sm_pool_blocks_kernel(const void* __restrict__ k_cache_,
                                                              const void* __restrict__ v_cache_, void* __restrict__ kp_,
                                                              void* __restrict__ vp_,
                                                              const int32_t* __restrict__ block_tables, int max_blocks,
-                                                             const int32_t* __restrict__ positions,
-                                                             const int32_t* __restrict__ tok_seq, int G, int D, int Dv,
+                                                             const int32_t* __restrict__ cu,
+                                                             const int32_t* __restrict__ positions, int G, int D, int Dv,
                                                              int bs, int pb, int pool) {
-  const int t = blockIdx.x, g = blockIdx.y;
-  const int pos = positions[t];
-  if ((pos + 1) % pool) return;
-  const int b = (pos + 1) / pool - 1;
-  const int32_t* bt = block_tables + (size_t)tok_seq[t] * max_blocks;
+  const int s = blockIdx.z, g = blockIdx.y;
+  const int lo = cu[s], n = cu[s + 1] - lo;
+  if (n <= 0) return;
+  const int start = positions[lo], end = start + n - 1;          // positions of the chunk's tokens
+  const int b = (start + pool) / pool - 1 + (int)blockIdx.x;     // first block whose last position is >= start
+  if ((long)b * pool + pool - 1 > end) return;
+  const int32_t* bt = block_tables + (size_t)s * max_blocks;
   const T* kc = (const T*)k_cache_;
   const T* vc = (const T*)v_cache_;
   const int pblk = bt[b / pb], poff = b % pb;
   T* kp = (T*)kp_ + (((size_t)pblk * G + g) * pb + poff) * D;
   T* vp = (T*)vp_ + ((size_t)pblk * G + g) * Dv * pb + poff;
   const float fpool = (float)pool;
-  for (int c = threadIdx.x; c < D + Dv; c += 128) {
-    float a = 0.f;
-    for (int j = b * pool; j < (b + 1) * pool; ++j) {
-      const int blk = bt[j / bs], off = j % bs;
-      a += c < D ? ldf(kc + (((size_t)blk * G + g) * bs + off) * D + c)
-                 : ldf(vc + (((size_t)blk * G + g) * Dv + (c - D)) * bs + off);
+  const int j0 = b * pool;
+  for (int c = threadIdx.x * V; c < D; c += 128 * V) {
+    float a[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) a[i] = 0.f;
+    for (int j = j0; j < j0 + pool; ++j) {
+      float x[V];
+      ldv<V>(kc + (((size_t)bt[j / bs] * G + g) * bs + j % bs) * D + c, x);
+#pragma unroll
+      for (int i = 0; i < V; ++i) a[i] += x[i];
     }
-    if (c < D) stf(kp + c, a / fpool);
-    else stf(vp + (size_t)(c - D) * pb, a / fpool);
+#pragma unroll
+    for (int i = 0; i < V; ++i) a[i] /= fpool;
+    stv<V>(kp + c, a);
+  }
+  for (int c = threadIdx.x; c < Dv; c += 128) {
+    float a = 0.f;
+    for (int j = j0; j < j0 + pool; ++j) a += ldf(vc + (((size_t)bt[j / bs] * G + g) * Dv + c) * bs + j % bs);
+    stf(vp + (size_t)c * pb, a / fpool);
   }
 }
 
 void sm_pool_blocks(uintptr_t k_cache, uintptr_t v_cache, uintptr_t kp_cache, uintptr_t vp_cache, uintptr_t block_tables,
-                    int max_blocks, uintptr_t positions, uintptr_t tok_seq, int tokens, int G, int D, int Dv, int bs,
-                    int pb, int pool, int f32, uintptr_t stream) {
-  if (tokens <= 0) return;
-  DLLM_HOST_CHECK(G > 0 && G <= 65535 && D > 0 && Dv > 0 && bs > 0 && pb > 0 && pool > 0 && (long)pb * pool >= bs &&
-                      max_blocks > 0 && k_cache && v_cache && kp_cache && vp_cache,
+                    int max_blocks, uintptr_t cu, uintptr_t positions, int seqs, int max_q_len, int G, int D, int Dv,
+                    int bs, int pb, int pool, int f32, uintptr_t stream) {
+  if (seqs <= 0 || max_q_len <= 0) return;
+  DLLM_HOST_CHECK(G > 0 && G <= 65535 && seqs <= 65535 && D > 0 && Dv > 0 && bs > 0 && pb > 0 && pool > 0 &&
+                      (long)pb * pool >= bs && max_blocks > 0 && k_cache && v_cache && kp_cache && vp_cache && cu && positions,
                   "pool_blocks arguments");
-  SM_DISPATCH(f32, sm_pool_blocks_kernel, dim3(tokens, G), dim3(128), 0, stream, (const void*)k_cache,
-              (const void*)v_cache, (void*)kp_cache, (void*)vp_cache, (const int32_t*)block_tables, max_blocks,
-              (const int32_t*)positions, (const int32_t*)tok_seq, G, D, Dv, bs, pb, pool);
+  const int esz = f32 ? 4 : 2;
+  const bool vec = D % 8 == 0 && k_cache % (8 * esz) == 0 && kp_cache % (8 * esz) == 0;
+  // a chunk of n tokens completes at most (n + pool - 1) / pool blocks
+  SM_DISPATCH_V(f32, vec, sm_pool_blocks_kernel, dim3((max_q_len + pool - 1) / pool, G, seqs), dim3(128), 0, stream,
+                (const void*)k_cache, (const void*)v_cache, (void*)kp_cache, (void*)vp_cache,
+                (const int32_t*)block_tables, max_blocks, (const int32_t*)cu, (const int32_t*)positions, G, D, Dv, bs, pb,
+                pool);
 }
 
 }  // namespace dllm

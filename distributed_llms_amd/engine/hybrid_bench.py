@@ -3,7 +3,9 @@ size (``bench.py --hybrid``), random weights, one GPU: Tudilix (sliding-window a
 a Llama-architecture model of the same width, layer count, feed-forward size, head size and K/V heads;
 Gikovik (latent attention + grouped-choice mixture of experts) beside a Mixtral-architecture model of the
 same width, layer count, heads, expert count and experts per token, with expert weights of equal size;
-Zebutar (chunked attention beside a gated delta rule, SwiGLU experts) beside the same Mixtral model.  Every step goes through the engine's StageRunner (the trace
+Zebutar (chunked attention beside a gated delta rule, SwiGLU experts) beside the same Mixtral model;
+Fekizen (window attention with averaged blocks beside gated linear attention, lightning layers, SwiGLU experts)
+beside the same Mixtral model and, for its kernels, beside Zebutar.  Every step goes through the engine's StageRunner (the trace
 replayer builds the batches): one step with ``batch`` prompts of ``prompt_len`` tokens (prefill),
 then ``gen_len`` steps of one token per sequence (decode)."""
 from __future__ import annotations
@@ -108,6 +110,31 @@ def zebutar_config(size: str, vocab: int = 32000) -> ModelConfig:
                                        "layers": layers}, name=f"zebutar-{size}")
 
 
+def fekizen_config(size: str, vocab: int = 32000) -> ModelConfig:
+    """Width, layers, heads, experts and experts per token of the Gikovik / Mixtral sizes.  Odd layers are
+    parallel: attention with the Mixtral model's heads (a quarter as many K/V heads, 128-wide, half of every
+    head rotated with blended frequencies, a window of 1024 positions plus one averaged key per 16 older
+    positions, capped scores, sinks) beside gated linear attention with as many 128 x 128 states as attention
+    heads; even layers are lightning attention with the same states.  Every layer has a mixture of three-matrix
+    experts of the Mixtral model's size with a shared expert; the first two layers are a loop that runs once
+    (its entry is part of the step)."""
+    w, nl, _ff, h, _d, _dr, _dv, _r, _qr, e, top, ef = GIKOVIK_SIZES[size]
+    inter = -(-(2 * ef // 3) // 256) * 256
+    moe = {"kind": "moe", "expert": {"ff": inter}, "shared": {"ff": inter}, "router": {"experts": e, "top": top}}
+    par = {"left": {"heads": h, "kv_heads": max(1, h // 4), "dim": 128, "vdim": 128, "mask": {"size": 1024, "pool": 16},
+                    "scale": 128 ** -0.5, "softcap": 50.0,
+                    "rot": {"base": 10000.0, "dims": 64,
+                            "scaling": {"factor": 4.0, "fast": 32.0, "original": 4096, "slow": 1.0}}},
+           "right": {"heads": h, "dim": 128, "vdim": 128, "tau": 16.0, "rank": 16}}
+    light = {"heads": h, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** -(3.0 + 6.0 * i / h) for i in range(h)]}
+    layers = [{"type": "parallel", "mixer": par, "mlp": moe} if i % 2 else {"type": "lightning", "mixer": light, "mlp": moe}
+              for i in range(nl)]
+    return ModelConfig.from_hf_config({"architecture": "Fekizen", "vocab": vocab, "width": w, "norm": {"eps": 1e-6},
+                                       "embedding": {"scale": float(w) ** 0.5}, "max_positions": 8192,
+                                       "loop": {"start": 0, "stop": 2, "times": 1}, "layers": layers},
+                                      name=f"fekizen-{size}")
+
+
 def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps: int, tmp: str, graphs: bool):
     import os
     os.makedirs(tmp, exist_ok=True)
@@ -145,14 +172,15 @@ def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps:
 
 
 MAKERS = {"tudilix": hybrid_config, "llama": llama_config, "gikovik": gikovik_config, "mixtral": mixtral_config,
-          "zebutar": zebutar_config}
-PAIRS = {"tudilix": "llama", "gikovik": "mixtral", "zebutar": "mixtral"}
+          "zebutar": zebutar_config, "fekizen": fekizen_config}
+PAIRS = {"tudilix": "llama", "gikovik": "mixtral", "zebutar": "mixtral", "fekizen": "mixtral"}
 
 
 def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int = 32, reps: int = 2,
         tmp: str = "/tmp/dllm_hybrid_bench", models=("tudilix", "llama")) -> dict:
-    """``models``: which to run, of tudilix, llama, gikovik, zebutar, mixtral; a layer-list model and its flat
-    counterpart (tudilix / llama, gikovik / mixtral, zebutar / mixtral) also get the ratio of their throughputs."""
+    """``models``: which to run, of tudilix, llama, gikovik, zebutar, fekizen, mixtral; a layer-list model and its
+    flat counterpart (tudilix / llama, gikovik / mixtral, zebutar / mixtral, fekizen / mixtral) also get the ratio
+    of their throughputs (``ratios`` holds every pair that ran; ``prefill_ratio`` / ``decode_ratio`` the first)."""
     out = {"size": size, "batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
            "data": "synthetic (random-init weights, random token ids)"}
     for key in models:
@@ -162,6 +190,9 @@ def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int 
                     "params_m": round(cfg.param_count() / 1e6, 1)}
     for a, b in PAIRS.items():
         if a in out and b in out:
-            out["prefill_ratio"] = round(out[a]["prefill_tok_s"] / out[b]["prefill_tok_s"], 3)
-            out["decode_ratio"] = round(out[a]["decode_tok_s"] / out[b]["decode_tok_s"], 3)
+            pr = round(out[a]["prefill_tok_s"] / out[b]["prefill_tok_s"], 3)
+            dr = round(out[a]["decode_tok_s"] / out[b]["decode_tok_s"], 3)
+            out.setdefault("ratios", {})[f"{a}/{b}"] = {"prefill": pr, "decode": dr}
+            out.setdefault("prefill_ratio", pr)
+            out.setdefault("decode_ratio", dr)
     return out

@@ -600,8 +600,8 @@ def pool_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, kp_cache: torch.Te
         _ck(c, n, k_cache.dtype)
     _ck(block_tables, "block_tables", torch.int32)
     _k().sm_pool_blocks(k_cache.data_ptr(), v_cache.data_ptr(), kp_cache.data_ptr(), vp_cache.data_ptr(),
-                        block_tables.data_ptr(), block_tables.shape[1], sb.positions.data_ptr(), sb.tok_seq.data_ptr(),
-                        sb.num_tokens, g, d, dv, bs, pb, int(pool), _f32flag(k_cache), _stream())
+                        block_tables.data_ptr(), block_tables.shape[1], sb.cu.data_ptr(), sb.positions.data_ptr(),
+                        sb.num_seqs, sb.max_q_len, g, d, dv, bs, pb, int(pool), _f32flag(k_cache), _stream())
 
 
 # ------------------------------------------------------------------ sliding-window attention

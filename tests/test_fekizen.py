@@ -434,7 +434,8 @@ def test_rotation_with_blended_frequencies_and_values_from_keys(target, shape):
 
 
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("sizes", [(3, 16, 24), (2, 48, 32), (1, 128, 128), (1, 8, 8), (2, 200, 20), (4, 20, 72), (2, 64, 130)])
+@pytest.mark.parametrize("sizes", [(3, 16, 24), (2, 48, 32), (1, 128, 128), (1, 8, 8), (2, 200, 20), (4, 20, 72), (2, 64, 130),
+                                   (1, 136, 72)])
 @pytest.mark.parametrize("mode", ["head", "channel"])
 def test_decayed_linear_attention_through_state_slots(target, sizes, mode):
     """S <- diag(a) S + k v^T, o = S^T q with a fixed decay per head (silu on q, k, v as they are read) or a decay
@@ -541,17 +542,17 @@ def test_mixer_outputs_normed_apart_then_averaged(target, width):
     xg, h = sm.mix_add(x.clone().to(device), o1.to(device), 1e-6)
     assert h is None
     np.testing.assert_allclose(xg.cpu().numpy(), d(x) + d(o1), atol=1e-5)
-    # gated norms: ``groups`` heads share w; one group = all heads normed together
-    hh, dv = 3, 8
-    o = torch.from_numpy((rng.standard_normal((t, hh * dv)) * np.repeat([9.0, 1.0, 0.1], dv)).astype(np.float32))
-    gate = T(rng.standard_normal((t, 5 + hh * dv)))
-    w_all, w_head = T(1 + 0.3 * rng.standard_normal(hh * dv)), T(1 + 0.3 * rng.standard_normal(dv))
-    y = la.gated_norm(o.to(device), gate.to(device), 5, w_all.to(device), 1e-6, groups=1, gate_act="sigmoid")
-    want = O.rms(d(o), 1e-6) * d(w_all) * O.sigmoid(d(gate)[:, 5:])
-    np.testing.assert_allclose(y.float().cpu().numpy(), want, atol=_atol(dtype, 2e-5, 4e-2) * np.abs(want).max())
-    y = la.gated_norm(o.to(device), gate.to(device), 5, w_head.to(device), 1e-6, groups=hh)
-    want = (O.rms(d(o).reshape(t, hh, dv), 1e-6) * d(w_head)).reshape(t, -1) * O.silu(d(gate)[:, 5:])
-    np.testing.assert_allclose(y.float().cpu().numpy(), want, atol=_atol(dtype, 2e-5, 4e-2) * np.abs(want).max())
+    # gated norms: ``groups`` heads share w; one group = all heads normed together (narrow, and wider than 512 channels)
+    for hh, dv in ((3, 8), (3, 264)):
+        o = torch.from_numpy((rng.standard_normal((t, hh * dv)) * np.repeat([9.0, 1.0, 0.1], dv)).astype(np.float32))
+        gate = T(rng.standard_normal((t, 8 + hh * dv)))
+        w_all, w_head = T(1 + 0.3 * rng.standard_normal(hh * dv)), T(1 + 0.3 * rng.standard_normal(dv))
+        y = la.gated_norm(o.to(device), gate.to(device), 8, w_all.to(device), 1e-6, groups=1, gate_act="sigmoid")
+        want = O.rms(d(o), 1e-6) * d(w_all) * O.sigmoid(d(gate)[:, 8:])
+        np.testing.assert_allclose(y.float().cpu().numpy(), want, atol=_atol(dtype, 2e-5, 4e-2) * np.abs(want).max())
+        y = la.gated_norm(o.to(device), gate.to(device), 8, w_head.to(device), 1e-6, groups=hh)
+        want = (O.rms(d(o).reshape(t, hh, dv), 1e-6) * d(w_head)).reshape(t, -1) * O.silu(d(gate)[:, 8:])
+        np.testing.assert_allclose(y.float().cpu().numpy(), want, atol=_atol(dtype, 2e-5, 4e-2) * np.abs(want).max())
 
 
 # ------------------------------------------------------------------------------ the engine
