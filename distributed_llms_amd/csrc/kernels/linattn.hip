@@ -238,7 +238,10 @@ void la_scan(uintptr_t o, uintptr_t proj, long ld, int qcol, int kcol, int vcol,
   // long chunks: four value columns per lane with the key channels over 8 lanes (a quarter of the LDS reads per
   // FMA; two columns for keys wider than 128, whose state would not fit the registers); short chunks (decode)
   // and narrow value heads: one column over 4 lanes, so that more workgroups share the state traffic
-  const bool wide = max_q_len >= 16 && Dv > 64;
+  // (also for long chunks of few sequences and heads: with four columns per lane they would leave most CUs idle,
+  // and the chain of one token's steps on a lone wave, not the arithmetic, bounds them)
+  const long wide_wgs = (long)seqs * H * ((Dv + 127) / 128);
+  const bool wide = max_q_len >= 16 && Dv > 64 && wide_wgs >= 256;
 #define LA_GO(T, DK, PARTS, CPL)                                                                                   \
   la_launch<T, DK, PARTS, CPL>(o, proj, ld, qcol, kcol, vcol, decay, z, z_bias, inv_tau, q_scale, silu, state, cu, \
                                positions, slots, seqs, H, D, Dv, stream)

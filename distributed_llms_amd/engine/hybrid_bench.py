@@ -122,10 +122,10 @@ def fekizen_config(size: str, vocab: int = 32000) -> ModelConfig:
     inter = -(-(2 * ef // 3) // 256) * 256
     moe = {"kind": "moe", "expert": {"ff": inter}, "shared": {"ff": inter}, "router": {"experts": e, "top": top}}
     par = {"left": {"heads": h, "kv_heads": max(1, h // 4), "dim": 128, "vdim": 128, "mask": {"size": 1024, "pool": 16},
-                    "scale": 128 ** -0.5, "softcap": 50.0,
+                    "scale": 128 ** -0.5, "softcap": 30.0,
                     "rot": {"base": 10000.0, "dims": 64,
                             "scaling": {"factor": 4.0, "fast": 32.0, "original": 4096, "slow": 1.0}}},
-           "right": {"heads": h, "dim": 128, "vdim": 128, "tau": 16.0, "rank": 16}}
+           "right": {"heads": h, "dim": 128, "vdim": 128, "tau": 8.0, "rank": 32}}
     light = {"heads": h, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** -(3.0 + 6.0 * i / h) for i in range(h)]}
     layers = [{"type": "parallel", "mixer": par, "mlp": moe} if i % 2 else {"type": "lightning", "mixer": light, "mlp": moe}
               for i in range(nl)]

@@ -54,7 +54,7 @@ from .hybrid import LayerListStage
 from .stage import BatchMeta
 from .weights import tensor_seed
 
-DEFAULT_DECAY_RANK = 16      # synthetic weights only: a checkpoint's tensors give the rank
+DEFAULT_DECAY_RANK = 8       # synthetic weights only: a checkpoint's tensors give the rank
 
 
 def layer_runs(cfg: ModelConfig) -> List[Tuple[int, Optional[int]]]:

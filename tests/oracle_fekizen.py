@@ -236,7 +236,7 @@ def shapes(cfg):
                       p + "mix.left.sink": (l["heads"],), p + "mix.left.o": (w, l["heads"] * l["vdim"]),
                       p + "mix.left.out": (w,), p + "mix.right.out": (w,)})
             qk, vv = r["heads"] * r["dim"], r["heads"] * r["vdim"]
-            rank = r.get("rank", 16)
+            rank = r.get("rank", 8)
             s.update({p + "mix.right.q": (qk, w), p + "mix.right.k": (qk, w), p + "mix.right.v": (vv, w),
                       p + "mix.right.g": (vv, w), p + "mix.right.o": (w, vv), p + "mix.right.norm": (r["vdim"],),
                       p + "mix.right.a1": (rank, w), p + "mix.right.a2": (qk, rank), p + "mix.right.a2.b": (qk,)})

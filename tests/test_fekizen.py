@@ -89,7 +89,7 @@ def cfg_c():
     return {"architecture": "Fekizen", "vocab": 160, "width": 128, "norm": {"eps": 1e-6}, "embedding": {"scale": 11.3},
             "max_positions": 512,
             "layers": [
-                _par(_left(4, 2, 64, 40, 8, 0.12, 50.0, 32, scaling=YARN), _right(2, 32, 128, 16.0), _moe(8, 2, 128, 128)),
+                _par(_left(4, 2, 64, 40, 8, 0.12, 40.0, 32, scaling=YARN), _right(2, 32, 128, 12.0), _moe(8, 2, 128, 128)),
                 _light(2, 64, 64, [0.8, 0.999], _moe(8, 2, 128, 128)),
                 _par(_left(4, 1, 32, 33, 16, 0.2, 15.0, 32), _right(1, 128, 64, 2.0), None),
             ]}
