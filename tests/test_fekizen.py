@@ -298,7 +298,7 @@ def _want_pooled_row(qq, kk, vv, p, h, g, size, pool, scale, cap, sink, kk_pool=
 
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("shape", [(4, 2, 24, 16, 20, 5), (6, 3, 64, 32, 72, 12), (3, 1, 16, 16, 9, 4), (2, 2, 32, 32, 33, 1),
-                                   (2, 1, 12, 32, 1, 1), (4, 4, 128, 32, 40, 33), (20, 1, 40, 32, 64, 7)])
+                                   (2, 1, 12, 32, 1, 1), (4, 4, 128, 32, 40, 33), (20, 1, 40, 32, 64, 7), (2, 1, 256, 32, 50, 6)])
 def test_window_with_averaged_blocks_capped_scores_and_a_sink(target, shape):
     """Attention over a window plus one mean key / value per block of older positions, with capped scores and a
     sink.  (a) Random inputs against the float64 rows: whole sequence, a late portion, decoded tokens; the
@@ -712,6 +712,32 @@ def test_drawn_models_on_a_mixed_schedule(target, seed, tmp_path):
     assert eng.bm.num_free() == eng.bm.num_blocks - 1
     for n, p in prompts.items():
         assert_close(got[n], oracle(cfg, sd, p), target, (seed, n))
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("case", ["lightning only", "parallel only, all looped", "no rotation, loop on the last layer"])
+def test_unusual_layer_orders(target, case, tmp_path):
+    """Models without attention caches at all, with every layer inside a loop of three passes, with a loop over
+    the last layer only and heads that do not turn: two requests in portions beside single tokens."""
+    base = {"architecture": "Fekizen", "vocab": 101, "width": 64, "norm": {"eps": 1e-6}, "embedding": {"scale": 4.0},
+            "max_positions": 128}
+    if case == "lightning only":
+        cfg = dict(base, layers=[_light(2, 16, 8, [0.9, 0.5], _moe(4, 2, 16, 16)), _light(1, 8, 24, [0.99], None)])
+    elif case == "parallel only, all looped":
+        cfg = dict(base, loop={"start": 0, "stop": 2, "times": 3},
+                   layers=[_par(_left(2, 1, 16, 6, 3, 0.2, 10.0, 8), _right(1, 8, 8, 2.0), None),
+                           _par(_left(2, 2, 8, 64, 2, 0.3, 5.0, 8), _right(2, 8, 16, 1.0, rank=2), _moe(3, 1, 8, 0))])
+    else:
+        cfg = dict(base, loop={"start": 2, "stop": 3, "times": 2},
+                   layers=[_light(2, 16, 8, [0.9, 0.5], None),
+                           _par(_left(4, 2, 16, 5, 7, 0.2, 10.0, 0), _right(1, 8, 8, 2.0), _moe(2, 2, 8, 8)),
+                           _light(1, 8, 8, [0.7], None)])
+    sd = _round(O.make_weights(cfg, seed=1), target[1])
+    eng = make_engine(cfg, sd, target, tmp_path, max_tokens=256, max_requests=3)
+    p = prompts_for(cfg, [70, 33], seed=2)
+    got = replay(eng, [[("r0", 40), ("r1", 2)], [("r0", 1), ("r1", 31)], [("r0", 29)]], p)
+    for n in p:
+        assert_close(got[n], oracle(cfg, sd, p[n]), target, (case, n))
 
 
 def test_config_round_trip_and_registry(tmp_path):
