@@ -2,8 +2,10 @@
 // with RMS norms before and after every sublayer, short causal convolutions whose tail lives in a
 // state slot, the real-gated linear recurrent unit (gates, then a chunked linear scan), the
 // attention input stages (convolution + per-head norm + interleaved rotation + paged append; whole-
-// projection norm + half-split rotation + paged append), embedding + norm, a clipped GLU and the logit
-// soft cap.
+// projection norm + half-split rotation + paged append), embedding (+ learned positions) + norm, the close of
+// pre-norm sublayers (one or two outputs, each normed apart), a token shift whose previous row lives in a state
+// slot, the entry of a looped span, the averaged keys / values of blocks of positions, a clipped GLU and the
+// logit soft cap.
 //
 // Every kernel is a template over the activation type T (bf16 or float): the float32 build is the
 // exact path (true 32-bit everywhere), the bf16 build keeps in float32 what feeds a norm, a

@@ -2,8 +2,11 @@
 pre- and post-sublayer RMS norms (also for sublayers that read the stream unnormed, and for two mixer
 outputs summed with scales), short causal convolutions with a state tail, the real-gated linear
 recurrent unit (RG-LRU), sliding-window and chunked attention over a paged K/V cache whose key and value
-widths differ, two attention input stages (convolution + per-head norm + interleaved rotation; whole-
-projection norm + half-split rotation), a clipped GLU and the logit soft cap.
+widths differ (optionally with capped scores, per-head sinks and one averaged key / value per block of
+positions older than the window), two attention input stages (convolution + per-head norm + interleaved
+rotation; whole-projection norm + half-split rotation, also without norms and with the values taken from
+the keys), the close of pre-norm sublayers whose outputs are normed apart, a token shift, the entry of a
+looped span of layers, a clipped GLU and the logit soft cap.
 
 Same dispatch as :mod:`distributed_llms_amd.ops`: a CUDA tensor goes to the in-tree HIP kernels
 (csrc/kernels/seqmix.hip, attention_window.hip) and raises if they are not built; CPU tensors run
